@@ -3,6 +3,9 @@
 
   * ``jax_llama_amd/_C*.so``   — the HIP kernels (``csrc/kernels/*.hip``, hipcc
     ``--offload-arch=gfx950``) + torch bindings (``csrc/bindings.cpp``);
+  * ``jax_llama_amd/_C_hybrid*.so`` — the hybrid-mixer kernels (``csrc/hybrid/*.hip``: row-gathered / expert-grouped
+    linears, biased soft-capped attention, the gated delta rule) + their bindings; small, self-contained, and the
+    only native code the hybrid model family needs (``--only hybrid`` builds it alone in about a minute);
   * ``jax_llama_amd/_bpe*.so`` — the C++ byte-pair-merge core of the Llama-3 tokenizer.
 
 The xGMI custom all-reduce (``csrc/kernels/allreduce.hip``) is part of ``_C``.
@@ -10,7 +13,7 @@ The xGMI custom all-reduce (``csrc/kernels/allreduce.hip``) is part of ``_C``.
 No hipify, no CUDA, no JIT cache: objects go to ``build/`` (incremental, mtime based) and the
 final ``.so`` files land next to the Python package so they travel with the repo snapshot.
 
-Usage: ``python build.py [-j N] [--force] [--only C|bpe] [--debug-bounds]``
+Usage: ``python build.py [-j N] [--force] [--only C|hybrid|bpe] [--debug-bounds]``
 
 ``--debug-bounds`` additionally builds ``jax_llama_amd/_C_dbg*.so`` (objects in ``build/C_dbg``) with
 ``-DJLA_DEBUG_BOUNDS``: every clamped / skipped out-of-range index that comes from device state (token ids,
@@ -67,7 +70,9 @@ def _stale(out: Path, deps) -> bool:
     return any(Path(d).stat().st_mtime > t for d in deps)
 
 
+# (no packed-fp32 VALU forms: the scalar fp32 instructions are used for all float code)
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-result", "-D__HIP_PLATFORM_AMD__"]
 
 
@@ -144,6 +149,44 @@ def build_C(jobs: int, force: bool, debug_bounds: bool = False) -> Path:
     return out
 
 
+def _compile_bindings(bsrc: Path, bobj: Path, headers, name: str, force: bool, extra=()):
+    _, tinc, _ = _torch_paths()
+    if force or _stale(bobj, [bsrc, *headers]):
+        bobj.parent.mkdir(parents=True, exist_ok=True)
+        inc = [f"-I{p}" for p in tinc] + [f"-I{_py_include()}", f"-I{CSRC}"]
+        _run([HIPCC, "-O2", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "--offload-host-only",
+              "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
+              f"-DTORCH_EXTENSION_NAME={name}", *extra, "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=1",
+              "-Wno-deprecated-declarations", "-Wno-unused-result", *inc, "-c", str(bsrc), "-o", str(bobj)])
+
+
+def _link(out: Path, objs, force: bool):
+    _, _, tlib = _torch_paths()
+    if force or _stale(out, objs):
+        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(out),
+              f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+              "-lamdhip64", f"-Wl,-rpath,{tlib}"])
+
+
+def build_hybrid(jobs: int, force: bool) -> Path:
+    """``_C_hybrid``: csrc/hybrid/*.hip + csrc/hybrid/bindings.cpp (its own module, so a hybrid model runs without
+    compiling the LLaMA kernels)."""
+    hdir = CSRC / "hybrid"
+    headers = sorted(hdir.glob("*.h")) + [CSRC / "kernels" / "common.h"]
+    srcs = sorted(hdir.glob("*.hip"))
+    odir = BUILD / "C_hybrid"
+    objs = [odir / (s.stem + ".o") for s in srcs]
+    bobj = odir / "bindings.o"
+    with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        futs = [ex.submit(_compile_hip, s, o, headers, force) for s, o in zip(srcs, objs)]
+        futs.append(ex.submit(_compile_bindings, hdir / "bindings.cpp", bobj, headers, "_C_hybrid", force))
+        for f in futs:
+            f.result()
+    out = PKG / f"_C_hybrid{EXT_SUFFIX}"
+    _link(out, [*objs, bobj], force)
+    return out
+
+
 def build_bpe(force: bool) -> Path:
     src = CSRC / "bpe" / "bpe.cpp"
     out = PKG / f"_bpe{EXT_SUFFIX}"
@@ -157,6 +200,8 @@ def build_all(jobs: int = 8, force: bool = False, only=None, debug_bounds: bool 
     outs = []
     if only in (None, "bpe"):
         outs.append(build_bpe(force))
+    if only in (None, "hybrid"):
+        outs.append(build_hybrid(jobs, force))
     if only in (None, "C"):
         outs.append(build_C(jobs, force))
         if debug_bounds:
@@ -168,7 +213,7 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=min(8, os.cpu_count() or 4))
     ap.add_argument("--force", action="store_true")
-    ap.add_argument("--only", choices=["C", "bpe"])
+    ap.add_argument("--only", choices=["C", "hybrid", "bpe"])
     ap.add_argument("--debug-bounds", action="store_true", help="also build the bounds-checked _C_dbg extension")
     a = ap.parse_args()
     for o in build_all(a.j, a.force, a.only, a.debug_bounds):

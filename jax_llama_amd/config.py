@@ -225,3 +225,153 @@ def get_preset(name: str, max_seq_len: Optional[int] = None, **overrides: Any) -
     for k, v in overrides.items():
         setattr(cfg, k, v)
     return cfg
+
+
+# -------------------------------------------------------------------------------------
+# Zavevik: a layer-list configuration (every layer names its mixer and its feed-forward)
+# -------------------------------------------------------------------------------------
+@dataclass
+class MixerSpec:
+    """One layer's sequence mixer. ``type`` ``"attention"``: softmax attention with RMS-normed q / k / v, an optional
+    query temperature (``q_temp_coef`` / ``q_temp_every``), score ``scale``, optional ``softcap`` and an optional
+    bucketed distance bias reaching ``bias_max``; ``kv_from``: the layer whose keys and values it reads instead of
+    projecting its own. ``type`` ``"delta"``: the gated delta rule with ``conv``-tap short convolutions."""
+
+    type: str
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int = 0
+    scale: float = 1.0
+    softcap: float = 0.0
+    bias_max: int = 0
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 1
+    kv_from: Optional[int] = None
+
+    @classmethod
+    def from_dict(cls, type_: str, d: Dict[str, Any]) -> "MixerSpec":
+        d = dict(d)
+        qt = d.pop("q_temp", None) or {}
+        known = dict(type=type_, heads=int(d.pop("heads")), kv_heads=int(d.pop("kv_heads")), dim=int(d.pop("dim")),
+                     vdim=int(d.pop("vdim")), conv=int(d.pop("conv", 0)), scale=float(d.pop("scale", 1.0)),
+                     softcap=float(d.pop("softcap", 0.0) or 0.0), bias_max=int(d.pop("bias_max", 0) or 0),
+                     q_temp_coef=float(qt.get("coef", 0.0)), q_temp_every=int(qt.get("every", 1)),
+                     kv_from=d.pop("kv_from", None))
+        if d:
+            raise ValueError(f"unknown mixer keys {sorted(d)}")
+        if known["kv_from"] is not None:
+            known["kv_from"] = int(known["kv_from"])
+        if type_ not in ("attention", "delta"):
+            raise ValueError(f"unknown mixer type {type_!r}")
+        if known["heads"] % known["kv_heads"]:
+            raise ValueError("heads must be divisible by kv_heads")
+        return cls(**known)
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = dict(heads=self.heads, kv_heads=self.kv_heads, dim=self.dim, vdim=self.vdim)
+        if self.type == "delta":
+            out["conv"] = self.conv
+            return out
+        out["scale"] = self.scale
+        if self.softcap:
+            out["softcap"] = self.softcap
+        if self.bias_max:
+            out["bias_max"] = self.bias_max
+        if self.q_temp_coef:
+            out["q_temp"] = {"coef": self.q_temp_coef, "every": self.q_temp_every}
+        if self.kv_from is not None:
+            out["kv_from"] = self.kv_from
+        return out
+
+
+@dataclass
+class MoESpec:
+    """Table-routed mixture of SwiGLU experts: ``experts`` experts of width ``ff``, ``top`` of them per token."""
+
+    experts: int
+    top: int
+    ff: int
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "MoESpec":
+        if d.get("kind", "moe") != "moe":
+            raise ValueError(f"unknown feed-forward kind {d.get('kind')!r}")
+        return cls(experts=int(d["router"]["experts"]), top=int(d["router"]["top"]), ff=int(d["expert"]["ff"]))
+
+    def to_dict(self) -> Dict[str, Any]:
+        return {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
+
+
+@dataclass
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: Optional[MoESpec]
+
+
+class ZavevikConfig:
+    """Zavevik decoder: ``config.json`` with ``architecture: "Zavevik"``, ``vocab``, ``width``, ``norm.eps``,
+    ``token_side.dim`` (optional) and a ``layers`` list of ``{type, mixer, mlp}`` entries."""
+
+    model_type = "zavevik"
+    architecture = "Zavevik"
+
+    def __init__(self, vocab_size: int, hidden_size: int, layers, norm_eps: float = 1e-6, side_dim: int = 0,
+                 pad_token_id: int = -1, eos_token_id: Optional[int] = None):
+        self.vocab_size = int(vocab_size)
+        self.hidden_size = int(hidden_size)
+        self.layers = list(layers)
+        self.norm_eps = float(norm_eps)
+        self.side_dim = int(side_dim)
+        self.pad_token_id = pad_token_id
+        self.eos_token_id = eos_token_id
+        for i, ls in enumerate(self.layers):
+            j = ls.mixer.kv_from
+            if j is not None:
+                src = self.layers[j].mixer if 0 <= j < i else None
+                if src is None or src.type != "attention" or src.kv_from is not None:
+                    raise ValueError(f"layer {i}: kv_from {j} is not an earlier attention layer with its own keys")
+                if (src.kv_heads, src.dim, src.vdim) != (ls.mixer.kv_heads, ls.mixer.dim, ls.mixer.vdim):
+                    raise ValueError(f"layer {i}: key / value geometry differs from layer {j}'s")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any]) -> "ZavevikConfig":
+        layers = [LayerSpec(MixerSpec.from_dict(e["type"], e["mixer"]),
+                            MoESpec.from_dict(e["mlp"]) if e.get("mlp") is not None else None) for e in d["layers"]]
+        side = d.get("token_side") or {}
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], layers=layers, norm_eps=d["norm"]["eps"],
+                   side_dim=side.get("dim", 0), pad_token_id=d.get("pad_token_id", -1),
+                   eos_token_id=d.get("eos_token_id"))
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+                               "norm": {"eps": self.norm_eps},
+                               "layers": [{"type": ls.mixer.type, "mixer": ls.mixer.to_dict(),
+                                           "mlp": ls.mlp.to_dict() if ls.mlp is not None else None}
+                                          for ls in self.layers]}
+        if self.side_dim:
+            out["token_side"] = {"dim": self.side_dim}
+        return out
+
+    def save_pretrained(self, save_directory: str) -> None:
+        os.makedirs(save_directory, exist_ok=True)
+        with open(os.path.join(save_directory, "config.json"), "w") as f:
+            json.dump(self.to_dict(), f, indent=1, sort_keys=True)
+
+    @classmethod
+    def from_pretrained(cls, path: str) -> "ZavevikConfig":
+        if os.path.isdir(path):
+            path = os.path.join(path, "config.json")
+        with open(path) as f:
+            return cls.from_dict(json.load(f))
+
+    def __eq__(self, other: object) -> bool:
+        return isinstance(other, ZavevikConfig) and self.to_dict() == other.to_dict()
+
+    def __repr__(self) -> str:
+        return f"ZavevikConfig {json.dumps(self.to_dict(), sort_keys=True)}"

@@ -1,0 +1,232 @@
+// Attention with per-head RMS-normalised q / k / v, a position-dependent query temperature, a soft cap on the scores
+// and a learned bias per key distance, over a per-layer cache of any head size (several layers may read one cache).
+//
+//   hy_attn_prep : from the fused projection output, per (token, head): divide q and k by their RMS over dim and v by
+//                  its RMS over vdim, scale q by 1 + coef * ln(floor((p + 1) / every) + 1), write k / v into the
+//                  cache at slot + s (bf16 or fp32), q to a dense fp32 buffer.
+//   hy_attn_bias : scores, soft cap, distance bias, causal softmax and PV in fp32. One wave per query (prefill) walks
+//                  its keys 64 at a time: a lane scores one key (q broadcast from LDS), the running maximum / sum are
+//                  wave reductions, and the lanes then split the value columns. Decode (S = 1) splits the keys of a
+//                  (row, head) over several waves whose partials a second kernel merges in split order.
+// The bias table is indexed by distance (rows past the last repeat it), so any bucketing is a host-side table fill.
+#include "hy_util.h"
+#include "hybrid.h"
+
+namespace jla {
+
+JLA_DEV float ab_ld(const float* p) { return *p; }
+JLA_DEV float ab_ld(const bf16_t* p) { return bf2f(*p); }
+JLA_DEV void ab_st(float* p, float v) { *p = v; }
+JLA_DEV void ab_st(bf16_t* p, float v) { *p = f2bf(v); }
+
+// grid (M, ceil(items / 4)), 4 waves: wave -> item: [0, H) q heads, [H, H + G) k heads, [H + G, H + 2G) v heads
+template <typename CT>
+__global__ void __launch_bounds__(256) attn_prep_kernel(AttnPrep p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = blockIdx.x, item = blockIdx.y * 4 + wave;
+  const int items = p.H + (p.has_kv ? 2 * p.G : 0);
+  if (item >= items) return;
+  const float* row = p.proj + (size_t)m * p.ld;
+  const int b = m / p.S, sidx = m - b * p.S;
+  int kind, head, len, col;
+  if (item < p.H) { kind = 0; head = item; len = p.dim; col = head * p.dim; }
+  else if (item < p.H + p.G) { kind = 1; head = item - p.H; len = p.dim; col = p.H * p.dim + head * p.dim; }
+  else { kind = 2; head = item - p.H - p.G; len = p.vdim; col = (p.H + p.G) * p.dim + head * p.vdim; }
+  float ss = 0.f;
+  for (int d = lane; d < len; d += 64) {
+    const float v = row[col + d];
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  float sc = 1.f / sqrtf(ss / (float)len + p.eps);
+  if (kind == 0) {
+    if (p.temp_coef != 0.f) {
+      const int pos = p.positions[m];
+      sc *= 1.f + p.temp_coef * logf((float)((pos + 1) / p.temp_every) + 1.f);
+    }
+    float* q = p.q + ((size_t)m * p.H + head) * p.dim;
+    for (int d = lane; d < len; d += 64) q[d] = row[col + d] * sc;
+    return;
+  }
+  const int t = *p.slot + sidx;
+  if (t < 0 || t >= p.T) return;  // cache full: the write is dropped
+  CT* dst = (kind == 1 ? reinterpret_cast<CT*>(p.kc) : reinterpret_cast<CT*>(p.vc)) +
+            (((size_t)b * p.G + head) * p.T + t) * len;
+  for (int d = lane; d < len; d += 64) ab_st(dst + d, row[col + d] * sc);
+}
+
+int hy_attn_prep(const AttnPrep& p, hipStream_t s) {
+  if (p.B < 0 || p.S < 1 || p.H < 1 || p.G < 1 || p.H % p.G || p.dim < 1 || p.vdim < 1 || p.T < 1) return -1;
+  if (p.temp_coef != 0.f && p.temp_every < 1) return -2;
+  const int M = p.B * p.S;
+  if (M == 0) return 0;
+  const int items = p.H + (p.has_kv ? 2 * p.G : 0);
+  if ((items + 3) / 4 > 65535) return -3;
+  dim3 grid(M, (items + 3) / 4);
+  if (p.cbf16) attn_prep_kernel<bf16_t><<<grid, 256, 0, s>>>(p);
+  else attn_prep_kernel<float><<<grid, 256, 0, s>>>(p);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+constexpr int AB_MAX_DIM = 512;   // q head held in LDS per wave
+constexpr int AB_MAX_VREG = 8;    // value columns per lane: vdim <= 512
+
+// One wave: keys [j_lo, j_hi) of query (b, h) at slot qi; returns the running max m, sum l and unnormalised acc.
+template <typename CT>
+JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, int j_lo, int j_hi, float& m_run,
+                     float& l_run, float* acc) {
+  const int lane = threadIdx.x & 63;
+  const int g = h / (p.H / p.G);
+  const CT* kbase = reinterpret_cast<const CT*>(p.kc) + ((size_t)b * p.G + g) * p.T * p.dim;
+  const CT* vbase = reinterpret_cast<const CT*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.vdim;
+  m_run = -INFINITY;
+  l_run = 0.f;
+#pragma unroll
+  for (int i = 0; i < AB_MAX_VREG; ++i) acc[i] = 0.f;
+  for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
+    const int j = j0 + lane;
+    float sc = -INFINITY;
+    if (j < j_hi) {
+      const CT* kr = kbase + (size_t)j * p.dim;
+      float d0 = 0.f, d1 = 0.f;
+      for (int d = 0; d < p.dim; d += 8) {
+        float kf[8];
+        hy_load8(kr + d, p.dim - d, kf);  // (zeros past dim)
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+          d0 = fmaf(d + i < p.dim ? qs[d + i] : 0.f, kf[i], d0);
+          d1 = fmaf(d + i + 1 < p.dim ? qs[d + i + 1] : 0.f, kf[i + 1], d1);
+        }
+      }
+      sc = (d0 + d1) * p.scale;
+      if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
+      if (p.bias) sc += p.bias[(size_t)min(qi - j, p.nbias - 1) * p.H + h];
+    }
+    const float m_new = fmaxf(m_run, wave_max(sc));
+    const float corr = expf(m_run - m_new);  // first chunk: exp(-inf) = 0
+    const float pr = j < j_hi ? expf(sc - m_new) : 0.f;
+    l_run = l_run * corr + wave_sum(pr);
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < AB_MAX_VREG; ++i) acc[i] *= corr;
+    const int nk = min(64, j_hi - j0);
+    for (int jj = 0; jj < nk; ++jj) {
+      const float pj = __shfl(pr, jj, 64);
+      const CT* vr = vbase + (size_t)(j0 + jj) * p.vdim;
+#pragma unroll
+      for (int i = 0; i < AB_MAX_VREG; ++i) {
+        const int c = lane + 64 * i;
+        if (c < p.vdim) acc[i] = fmaf(pj, ab_ld(vr + c), acc[i]);
+      }
+    }
+  }
+}
+
+// prefill: grid (ceil(S / 4), H, B), one wave per query
+template <typename CT>
+__global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
+  __shared__ float qs_all[4][AB_MAX_DIM];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int s = blockIdx.x * 4 + wave, h = blockIdx.y, b = blockIdx.z;
+  if (s >= p.S) return;
+  float* qs = qs_all[wave];
+  const float* q = p.q + (((size_t)b * p.S + s) * p.H + h) * p.dim;
+  for (int d = lane; d < p.dim; d += 64) qs[d] = q[d];
+  __builtin_amdgcn_wave_barrier();
+  const int qi = min(*p.slot + s, p.T - 1);
+  float m_run, l_run, acc[AB_MAX_VREG];
+  ab_wave<CT>(p, qs, b, h, qi, 0, qi + 1, m_run, l_run, acc);
+  float* o = p.out + ((size_t)b * p.S + s) * (p.H * p.vdim) + (size_t)h * p.vdim;
+  const float inv = 1.f / l_run;
+#pragma unroll
+  for (int i = 0; i < AB_MAX_VREG; ++i) {
+    const int c = lane + 64 * i;
+    if (c < p.vdim) o[c] = acc[i] * inv;
+  }
+}
+
+// decode: grid (splits, H, B), one wave per (row, head, split); partial = [m, l, acc[vdim]]
+template <typename CT>
+__global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
+  __shared__ float qs[AB_MAX_DIM];
+  const int lane = threadIdx.x;
+  const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const float* q = p.q + ((size_t)b * p.H + h) * p.dim;
+  for (int d = lane; d < p.dim; d += 64) qs[d] = q[d];
+  __syncthreads();
+  const int qi = min(*p.slot, p.T - 1);
+  const int n = qi + 1;
+  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
+  const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
+  float m_run, l_run, acc[AB_MAX_VREG];
+  ab_wave<CT>(p, qs, b, h, qi, j_lo, j_hi, m_run, l_run, acc);
+  float* w = p.ws + (((size_t)b * p.H + h) * p.splits + sp) * (p.vdim + 2);
+  if (lane == 0) {
+    w[0] = m_run;
+    w[1] = l_run;
+  }
+#pragma unroll
+  for (int i = 0; i < AB_MAX_VREG; ++i) {
+    const int c = lane + 64 * i;
+    if (c < p.vdim) w[2 + c] = acc[i];
+  }
+}
+
+// grid (H, B), 64 threads: merge the splits in order
+__global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
+  const int lane = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
+  const float* w = p.ws + ((size_t)b * p.H + h) * p.splits * (p.vdim + 2);
+  float m = -INFINITY;
+  for (int sp = 0; sp < p.splits; ++sp) m = fmaxf(m, w[(size_t)sp * (p.vdim + 2)]);
+  float l = 0.f;
+  for (int sp = 0; sp < p.splits; ++sp) {
+    const float* ws = w + (size_t)sp * (p.vdim + 2);
+    if (ws[1] > 0.f) l += ws[1] * expf(ws[0] - m);
+  }
+  float* o = p.out + (size_t)b * (p.H * p.vdim) + (size_t)h * p.vdim;
+  for (int c = lane; c < p.vdim; c += 64) {
+    float a = 0.f;
+    for (int sp = 0; sp < p.splits; ++sp) {
+      const float* ws = w + (size_t)sp * (p.vdim + 2);
+      if (ws[1] > 0.f) a += ws[2 + c] * expf(ws[0] - m);
+    }
+    o[c] = a / l;
+  }
+}
+
+int hy_attn_decode_splits(int B, int H, int t_cap) {
+  // enough waves for the chip (256 CUs x 4 SIMDs), at least 256 keys per split
+  const long long pairs = (long long)B * H;
+  long long want = (2048 + pairs - 1) / (pairs > 0 ? pairs : 1);
+  const long long by_len = (t_cap + 255) / 256;
+  if (want > by_len) want = by_len;
+  if (want < 1) want = 1;
+  if (want > 64) want = 64;
+  return (int)want;
+}
+
+int hy_attn_bias(const AttnBias& p, hipStream_t s) {
+  if (p.B < 0 || p.S < 1 || p.H < 1 || p.G < 1 || p.H % p.G || p.T < 1) return -1;
+  if (p.dim < 1 || p.dim > AB_MAX_DIM || p.vdim < 1 || p.vdim > 64 * AB_MAX_VREG) return -2;
+  if (p.bias && p.nbias < 1) return -3;
+  if (p.B == 0) return 0;
+  if (p.H > 65535 || p.B > 65535) return -4;
+  if (p.S == 1) {
+    if (p.splits < 1 || !p.ws) return -5;
+    dim3 grid(p.splits, p.H, p.B);
+    if (p.cbf16) attn_bias_decode_kernel<bf16_t><<<grid, 64, 0, s>>>(p);
+    else attn_bias_decode_kernel<float><<<grid, 64, 0, s>>>(p);
+    JLA_CHECK_LAUNCH();
+    attn_bias_merge_kernel<<<dim3(p.H, p.B), 64, 0, s>>>(p);
+    JLA_CHECK_LAUNCH();
+    return 0;
+  }
+  dim3 grid((p.S + 3) / 4, p.H, p.B);
+  if (p.cbf16) attn_bias_prefill_kernel<bf16_t><<<grid, 256, 0, s>>>(p);
+  else attn_bias_prefill_kernel<float><<<grid, 256, 0, s>>>(p);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace jla

@@ -1,0 +1,282 @@
+// Row-gathered, expert-grouped linear on row-major weights of any shape (no N % 16 / K % 32 packing constraint):
+//   out[dst(r), :] = act(A[src(r), :] @ W[expert(r)]^T)
+// A is fp32 in memory. With bf16 weights the A tile is rounded to bf16 while it is staged (v_mfma_f32_32x32x16_bf16,
+// fp32 accumulation); with fp32 weights everything stays fp32 on the exact-f32 MFMA (v_mfma_f32_32x32x2_f32).
+//
+//  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS. With an
+//    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
+//    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
+//  * few rows (decode): one wave per output column streams the weight row once and dots it with up to 8 rows.
+//  * swiglu epilogue: the gate and the up rows of a column are accumulated side by side, out = silu(g) * u.
+// The table router's counting sort is here too.
+#include "hy_util.h"
+#include "hybrid.h"
+
+namespace jla {
+
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+
+constexpr int LR_BM = 64, LR_BN = 64, LR_BK = 32, LR_THREADS = 256;
+
+template <typename WT>
+struct LrTile;
+template <>
+struct LrTile<bf16_t> {
+  static constexpr int LD = LR_BK + 8;  // 80-byte rows: 16-byte aligned fragment reads, rows spread over the banks
+};
+template <>
+struct LrTile<float> {
+  static constexpr int LD = LR_BK + 1;
+};
+
+JLA_DEV void lr_store8(bf16_t* dst, const float* f) { *reinterpret_cast<u32x4*>(dst) = pack8(f); }
+JLA_DEV void lr_store8(float* dst, const float* f) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) dst[i] = f[i];
+}
+
+JLA_DEV void lr_mma(const bf16_t* a_row, const bf16_t* b_row, int hi, f32x16& acc) {
+#pragma unroll
+  for (int kk = 0; kk < LR_BK / 16; ++kk) {
+    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(a_row + 16 * kk + 8 * hi);
+    const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(b_row + 16 * kk + 8 * hi);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+  }
+}
+JLA_DEV void lr_mma(const float* a_row, const float* b_row, int hi, f32x16& acc) {
+#pragma unroll
+  for (int kk = 0; kk < LR_BK / 2; ++kk)
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_row[2 * kk + hi], b_row[2 * kk + hi], acc, 0, 0, 0);
+}
+
+template <typename WT, int SWIGLU>
+__global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
+  constexpr int LD = LrTile<WT>::LD;
+  __shared__ __attribute__((aligned(16))) WT As[LR_BM * LD];
+  __shared__ __attribute__((aligned(16))) WT Bs[(SWIGLU ? 2 : 1) * LR_BN * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, hi = lane >> 5;
+  // which expert and which rows
+  int e = 0, r0 = blockIdx.y * LR_BM, rend = p.R;
+  if (p.offs) {
+    int tile = blockIdx.y;
+    bool found = false;
+    for (e = 0; e < p.E; ++e) {
+      const int b = p.offs[e], cnt = p.offs[e + 1] - b, nt = (cnt + LR_BM - 1) / LR_BM;
+      if (tile < nt) {
+        r0 = b + tile * LR_BM;
+        rend = b + cnt;
+        found = true;
+        break;
+      }
+      tile -= nt;
+    }
+    if (!found) return;
+  } else if (r0 >= rend) {
+    return;
+  }
+  const int n0 = blockIdx.x * LR_BN;
+  const WT* W = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride;
+  const int K = p.K, N = p.N;
+
+  // staging role: 8 consecutive k of one row
+  const int srow = tid >> 2, skq = (tid & 3) * 8;
+  const int ar = r0 + srow;
+  const float* a_ptr = nullptr;
+  if (ar < rend) a_ptr = p.a + (size_t)(p.a_idx ? p.a_idx[ar] : ar) * p.lda;
+  const int wr = n0 + srow;
+  const WT* w_ptr = wr < N ? W + (size_t)wr * K : nullptr;
+  const WT* w2_ptr = (SWIGLU && wr < N) ? W + (size_t)(N + wr) * K : nullptr;
+
+  f32x16 acc, acc2;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += LR_BK) {
+    const int gk = k0 + skq, left = K - gk;
+    float f[8];
+    if (a_ptr && left > 0) hy_load8(a_ptr + gk, left, f);
+    else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = 0.f;
+    }
+    lr_store8(&As[srow * LD + skq], f);
+    if (w_ptr && left > 0) hy_load8(w_ptr + gk, left, f);
+    else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = 0.f;
+    }
+    lr_store8(&Bs[srow * LD + skq], f);
+    if (SWIGLU) {
+      if (w2_ptr && left > 0) hy_load8(w2_ptr + gk, left, f);
+      else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = 0.f;
+      }
+      lr_store8(&Bs[(LR_BN + srow) * LD + skq], f);
+    }
+    __syncthreads();
+    const WT* a_row = &As[(wm * 32 + (lane & 31)) * LD];
+    const WT* b_row = &Bs[(wn * 32 + (lane & 31)) * LD];
+    lr_mma(a_row, b_row, hi, acc);
+    if (SWIGLU) lr_mma(a_row, b_row + LR_BN * LD, hi, acc2);
+    __syncthreads();
+  }
+  // C/D map of the 32 x 32 shapes: col = lane & 31, row = (r & 3) + 8 (r >> 2) + 4 (lane >> 5)
+  const int col = n0 + wn * 32 + (lane & 31);
+  if (col >= N) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = r0 + wm * 32 + (r & 3) + 8 * (r >> 2) + 4 * hi;
+    if (row < rend) {
+      const int drow = p.dst_idx ? p.dst_idx[row] : row;
+      p.out[(size_t)drow * p.ldo + col] = SWIGLU ? hy_silu(acc[r]) * acc2[r] : acc[r];
+    }
+  }
+}
+
+JLA_DEV float lr_round(float v, const bf16_t*) { return bf2f(f2bf(v)); }
+JLA_DEV float lr_round(float v, const float*) { return v; }
+
+// One wave per output column; rows [g * MAXR, ...) of group g = blockIdx.y (row_expert: one row per group).
+template <typename WT, int SWIGLU>
+__global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int rows_per_group) {
+  constexpr int MAXR = HY_GEMV_MAX_R;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * (LR_THREADS / 64) + wave;
+  if (n >= p.N) return;
+  const int r0 = blockIdx.y * rows_per_group;
+  const int nr = min(rows_per_group, p.R - r0);
+  if (nr <= 0) return;
+  const int e = p.row_expert ? p.row_expert[r0] : 0;
+  const int K = p.K;
+  const WT* w = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride + (size_t)n * K;
+  const WT* w2 = w + (size_t)p.N * K;
+  const float* a[MAXR];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    const int rr = r0 + min(r, nr - 1);
+    a[r] = p.a + (size_t)(p.a_idx ? p.a_idx[rr] : rr) * p.lda;
+  }
+  float acc[MAXR], acc2[MAXR];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) acc[r] = acc2[r] = 0.f;
+  for (int k = lane * 8; k < K; k += 64 * 8) {
+    const int left = K - k;
+    float wf[8], uf[8], xf[8];
+    hy_load8(w + k, left, wf);
+    if (SWIGLU) hy_load8(w2 + k, left, uf);
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      if (r < nr) {
+        hy_load8(a[r] + k, left, xf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xv = lr_round(xf[i], w);
+          acc[r] = fmaf(xv, wf[i], acc[r]);
+          if (SWIGLU) acc2[r] = fmaf(xv, uf[i], acc2[r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < nr) {  // (wave-uniform)
+      const float g = wave_sum(acc[r]);
+      const float u = SWIGLU ? wave_sum(acc2[r]) : 0.f;
+      if (lane == 0) {
+        const int row = r0 + r, drow = p.dst_idx ? p.dst_idx[row] : row;
+        p.out[(size_t)drow * p.ldo + n] = SWIGLU ? hy_silu(g) * u : g;
+      }
+    }
+  }
+}
+
+int hy_linear_rows(const RowLinear& p, hipStream_t s) {
+  if (p.R < 0 || p.N <= 0 || p.K <= 0 || p.lda < p.K || p.ldo < p.N || p.E < 1) return -1;
+  if (p.R == 0) return 0;
+  if (p.offs && p.E > 65535) return -2;
+  const bool small = p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert);
+  if (small) {
+    const int rpg = p.row_expert ? 1 : HY_GEMV_MAX_R;
+    dim3 grid((p.N + 3) / 4, (p.R + rpg - 1) / rpg);
+    RowLinear q = p;
+    q.offs = nullptr;
+    if (p.wbf16) {
+      if (p.swiglu) lr_gemv_kernel<bf16_t, 1><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+      else lr_gemv_kernel<bf16_t, 0><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+    } else {
+      if (p.swiglu) lr_gemv_kernel<float, 1><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+      else lr_gemv_kernel<float, 0><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+    }
+    JLA_CHECK_LAUNCH();
+    return 0;
+  }
+  if (!p.offs && p.E != 1) return -3;
+  const long long mt = (p.R + LR_BM - 1) / LR_BM + (p.offs ? p.E : 0);
+  if (mt > 65535) return -4;
+  dim3 grid((p.N + LR_BN - 1) / LR_BN, (unsigned)mt);
+  RowLinear q = p;
+  q.row_expert = nullptr;
+  if (p.wbf16) {
+    if (p.swiglu) lr_gemm_kernel<bf16_t, 1><<<grid, LR_THREADS, 0, s>>>(q);
+    else lr_gemm_kernel<bf16_t, 0><<<grid, LR_THREADS, 0, s>>>(q);
+  } else {
+    if (p.swiglu) lr_gemm_kernel<float, 1><<<grid, LR_THREADS, 0, s>>>(q);
+    else lr_gemm_kernel<float, 0><<<grid, LR_THREADS, 0, s>>>(q);
+  }
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+// ---- table router: counting sort of the (token, choice) rows by expert (one workgroup) -------------------------------
+constexpr int RT_MAX_E = 1024;
+
+__global__ void __launch_bounds__(256) route_table_kernel(const int32_t* ids, const int32_t* table, int V, int M, int top,
+                                                          int E, int32_t* row_expert, int32_t* row_tok,
+                                                          int32_t* sort_tok, int32_t* sort_dst, int32_t* offs) {
+  __shared__ int cnt[RT_MAX_E + 1];
+  __shared__ int cur[RT_MAX_E];
+  const int R = M * top;
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int r = threadIdx.x; r < R; r += blockDim.x) {
+    const int m = r / top, c = r - m * top;
+    int id = ids[m];
+    id = id < 0 || id >= V ? 0 : id;
+    int e = table[(size_t)id * top + c];
+    e = e < 0 || e >= E ? 0 : e;
+    row_expert[r] = e;
+    row_tok[r] = m;
+    atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cnt[e];
+      cur[e] = run;
+      offs[e] = run;
+      run += c;
+    }
+    offs[E] = run;
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < R; r += blockDim.x) {
+    const int e = row_expert[r];
+    const int pos = atomicAdd(&cur[e], 1);
+    sort_tok[pos] = r / top;
+    sort_dst[pos] = r;
+  }
+}
+
+int hy_route_table(const int32_t* ids, const int32_t* table, int V, int M, int top, int E, int32_t* row_expert,
+                   int32_t* row_tok, int32_t* sort_tok, int32_t* sort_dst, int32_t* offs, hipStream_t s) {
+  if (M < 0 || top < 1 || E < 1 || E > RT_MAX_E || V < 1) return -1;
+  if (M == 0) return 0;
+  route_table_kernel<<<1, 256, 0, s>>>(ids, table, V, M, top, E, row_expert, row_tok, sort_tok, sort_dst, offs);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace jla

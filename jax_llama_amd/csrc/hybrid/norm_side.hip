@@ -1,0 +1,92 @@
+// Row kernels of the hybrid stack: embedding-slice gather, the norm on a sublayer's OUTPUT fused with the residual add
+// (x += rms_norm(sum of the chosen experts' outputs) * w, w one number or a vector), and the per-layer token-side gate
+// (gelu_tanh(gate projection) * a slice of a second embedding table). fp32 statistics and residual.
+#include "hy_util.h"
+#include "hybrid.h"
+
+namespace jla {
+
+JLA_DEV float ns_ld(const float* p) { return *p; }
+JLA_DEV float ns_ld(const bf16_t* p) { return bf2f(*p); }
+
+template <typename WT>
+__global__ void __launch_bounds__(256) embed_rows_kernel(const int32_t* ids, const WT* table, int V, int ld, int col0,
+                                                         float* out, int D) {
+  const int m = blockIdx.x;
+  int id = ids[m];
+  id = id < 0 || id >= V ? 0 : id;
+  const WT* row = table + (size_t)id * ld + col0;
+  for (int d = threadIdx.x; d < D; d += 256) out[(size_t)m * D + d] = ns_ld(row + d);
+}
+
+int hy_embed_rows(const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0, float* out, int M, int D,
+                  hipStream_t s) {
+  if (M < 0 || D < 1 || V < 1 || col0 < 0 || col0 + D > ld) return -1;
+  if (M == 0) return 0;
+  if (wbf16) embed_rows_kernel<bf16_t><<<M, 256, 0, s>>>(ids, reinterpret_cast<const bf16_t*>(table), V, ld, col0, out, D);
+  else embed_rows_kernel<float><<<M, 256, 0, s>>>(ids, reinterpret_cast<const float*>(table), V, ld, col0, out, D);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+// one workgroup per row
+__global__ void __launch_bounds__(256) norm_residual_kernel(const float* y, int nsum, float ysc, const float* w,
+                                                            int w_vec, float eps, float* x, float* out, int D) {
+  __shared__ float red[16];
+  const int m = blockIdx.x;
+  const float* yr = y + (size_t)m * nsum * D;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    float v = 0.f;
+    for (int c = 0; c < nsum; ++c) v += yr[(size_t)c * D + d];
+    v *= ysc;
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float sc = 1.f / sqrtf(ss / (float)D + eps);
+  const float w0 = w_vec ? 0.f : w[0];
+  for (int d = threadIdx.x; d < D; d += 256) {
+    float v = 0.f;
+    for (int c = 0; c < nsum; ++c) v += yr[(size_t)c * D + d];
+    v = v * ysc * sc * (w_vec ? w[d] : w0);
+    if (x) x[(size_t)m * D + d] += v;
+    else out[(size_t)m * D + d] = v;
+  }
+}
+
+int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_vec, float eps, float* x, float* out,
+                     int M, int D, hipStream_t s) {
+  if (M < 0 || D < 1 || nsum < 1 || (!x && !out)) return -1;
+  if (M == 0) return 0;
+  norm_residual_kernel<<<M, 256, 0, s>>>(y, nsum, ysc, w, w_vec, eps, x, out, D);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+JLA_DEV float ns_gelu_tanh(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename WT>
+__global__ void __launch_bounds__(256) gelu_gate_rows_kernel(const float* gp, const int32_t* ids, const WT* table, int V,
+                                                             int ld, int col0, float* g, int D) {
+  const int m = blockIdx.x;
+  int id = ids[m];
+  id = id < 0 || id >= V ? 0 : id;
+  const WT* row = table + (size_t)id * ld + col0;
+  for (int d = threadIdx.x; d < D; d += 256) g[(size_t)m * D + d] = ns_gelu_tanh(gp[(size_t)m * D + d]) * ns_ld(row + d);
+}
+
+int hy_gelu_gate_rows(const float* gp, const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0,
+                      float* g, int M, int D, hipStream_t s) {
+  if (M < 0 || D < 1 || V < 1 || col0 < 0 || col0 + D > ld) return -1;
+  if (M == 0) return 0;
+  if (wbf16)
+    gelu_gate_rows_kernel<bf16_t><<<M, 256, 0, s>>>(gp, ids, reinterpret_cast<const bf16_t*>(table), V, ld, col0, g, D);
+  else
+    gelu_gate_rows_kernel<float><<<M, 256, 0, s>>>(gp, ids, reinterpret_cast<const float*>(table), V, ld, col0, g, D);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace jla

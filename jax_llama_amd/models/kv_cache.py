@@ -43,6 +43,12 @@ class KVCache:
         self.index = 0
         self.index_t.zero_()
 
+    def clear(self) -> None:
+        """``reset`` and zero the keys and values (after a failed step may have left non-finite rows)."""
+        self.reset()
+        self.k.zero_()
+        self.v.zero_()
+
     def rows(self, b0: int, b1: int) -> "KVCacheRows":
         """The cache of batch rows ``[b0, b1)`` (every layer): a view whose per-layer K / V are contiguous slices, for a
         prefill run in row chunks (runtime/engine.py)."""
@@ -87,3 +93,137 @@ class KVCacheRows:
 
     def layer(self, i: int):
         return self.parent.k[i, self.b0:self.b1], self.parent.v[i, self.b0:self.b1]
+
+
+class HybridCache:
+    """Per-layer sequence state of a stack that mixes attention and recurrent layers, pre-allocated.
+
+    ``specs[i]`` describes layer ``i``:
+      * ``("kv", kv_heads, dim, vdim)``: keys ``[B, G, T, dim]`` and values ``[B, G, T, vdim]`` (head sizes are per
+        layer, keys and values may differ in width);
+      * ``("kv_from", j)``: no storage, ``layer(i)`` is layer ``j``'s keys and values (cross-layer KV sharing);
+      * ``("delta", heads, kv_heads, dim, vdim, taps)``: a recurrent state ``[B, H, dim, vdim]`` (always fp32) and
+        the short convolutions' input tail ``[B, 2 G dim + H vdim, taps - 1]`` (fp32);
+      * ``None``: nothing.
+    The slot index (tokens held, the same for every row) is mirrored on the device like ``KVCache``'s, so captured
+    decode steps advance it without the host. ``dtype`` is the key / value element type (bf16, or fp32 for exact runs).
+    Recurrent state has no slot: ``reset`` zeroes it, since a new sequence starts from a zero state."""
+
+    def __init__(self, specs, batch_size: int, max_length: int, device, dtype=torch.bfloat16):
+        device = torch.device(device)
+        self.specs = list(specs)
+        self.batch_size = batch_size
+        self.max_length = max_length
+        self.dtype = dtype
+        self._k, self._v, self._state, self._conv = {}, {}, {}, {}
+        for i, sp in enumerate(self.specs):
+            if sp is None:
+                continue
+            if sp[0] == "kv":
+                _, g, dim, vdim = sp
+                self._k[i] = torch.zeros(batch_size, g, max_length, dim, dtype=dtype, device=device)
+                self._v[i] = torch.zeros(batch_size, g, max_length, vdim, dtype=dtype, device=device)
+            elif sp[0] == "kv_from":
+                j = sp[1]
+                if not (0 <= j < i) or self.specs[j] is None or self.specs[j][0] != "kv":
+                    raise ValueError(f"layer {i} shares the keys / values of layer {j}, which holds none before it")
+            elif sp[0] == "delta":
+                _, h, g, dim, vdim, taps = sp
+                self._state[i] = torch.zeros(batch_size, h, dim, vdim, dtype=torch.float32, device=device)
+                self._conv[i] = torch.zeros(batch_size, 2 * g * dim + h * vdim, max(taps - 1, 0),
+                                            dtype=torch.float32, device=device)
+            else:
+                raise ValueError(f"unknown cache spec {sp!r}")
+        self._device = device
+        self.index = 0
+        self.index_t = torch.zeros(1, dtype=torch.int32, device=device)
+
+    @property
+    def device(self):
+        return self._device
+
+    def layer(self, i: int):
+        """Keys and values layer ``i`` attends over (its own, or the layer's it shares them with)."""
+        sp = self.specs[i]
+        j = sp[1] if sp[0] == "kv_from" else i
+        return self._k[j], self._v[j]
+
+    def owns_kv(self, i: int) -> bool:
+        return self.specs[i] is not None and self.specs[i][0] == "kv"
+
+    def recurrent(self, i: int):
+        """``(state, conv tail)`` of a recurrent layer."""
+        return self._state[i], self._conv[i]
+
+    def advance(self, n: int) -> None:
+        self.index += n
+        self.index_t.add_(n)
+
+    def reset(self) -> None:
+        """Empty: slot 0, zero recurrent state (keys and values past the slot are never read)."""
+        self.index = 0
+        self.index_t.zero_()
+        for t in list(self._state.values()) + list(self._conv.values()):
+            t.zero_()
+
+    def clear(self) -> None:
+        """``reset`` and zero the keys and values too (after a failed step may have left non-finite rows)."""
+        self.reset()
+        for t in list(self._k.values()) + list(self._v.values()):
+            t.zero_()
+
+    def rows(self, b0: int, b1: int) -> "HybridCacheRows":
+        return HybridCacheRows(self, b0, b1)
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for d in (self._k, self._v, self._state, self._conv)
+                   for t in d.values())
+
+    @staticmethod
+    def bytes_per(specs, batch_size: int, max_length: int, dtype=torch.bfloat16) -> int:
+        """Bytes a cache of this geometry takes (without allocating it)."""
+        es = torch.empty(0, dtype=dtype).element_size()
+        n = 0
+        for sp in specs:
+            if sp is None or sp[0] == "kv_from":
+                continue
+            if sp[0] == "kv":
+                n += batch_size * sp[1] * max_length * (sp[2] + sp[3]) * es
+            else:
+                _, h, g, dim, vdim, taps = sp
+                n += 4 * batch_size * (h * dim * vdim + (2 * g * dim + h * vdim) * max(taps - 1, 0))
+        return n
+
+
+class HybridCacheRows:
+    """Rows ``[b0, b1)`` of a HybridCache (contiguous slices of every tensor; the slot index is the parent's)."""
+
+    def __init__(self, parent: HybridCache, b0: int, b1: int):
+        self.parent = parent
+        self.b0, self.b1 = b0, b1
+        self.batch_size = b1 - b0
+        self.max_length = parent.max_length
+        self.specs = parent.specs
+
+    @property
+    def device(self):
+        return self.parent.device
+
+    @property
+    def index(self):
+        return self.parent.index
+
+    @property
+    def index_t(self):
+        return self.parent.index_t
+
+    def layer(self, i: int):
+        k, v = self.parent.layer(i)
+        return k[self.b0:self.b1], v[self.b0:self.b1]
+
+    def owns_kv(self, i: int) -> bool:
+        return self.parent.owns_kv(i)
+
+    def recurrent(self, i: int):
+        s, c = self.parent.recurrent(i)
+        return s[self.b0:self.b1], c[self.b0:self.b1]
