@@ -166,7 +166,7 @@ class DecodeEngine:
         if self.device.type == "cuda":
             ops.ext().decode_update(nxt, self.finished, self.sequences, self.cur_len, self.tokens,
                                     self.positions, self.cache.index_t, int(self.gc.pad_token_id),
-                                    int(self.gc.eos_token_id))
+                                    int(self.gc.eos_token_id))  # (eos -1: a model without an end token never finishes)
             return
         fin = self.finished.bool()
         nxt = torch.where(fin, torch.full_like(nxt, self.gc.pad_token_id), nxt)
@@ -306,8 +306,7 @@ class DecodeEngine:
             # a failed step (a peer or in-launch timeout, an error mid-decode) can leave non-finite rows in this
             # engine's cache beyond where the next prompt writes; the kernels mask keys past the valid length by
             # probability 0, and 0 x NaN is NaN: zero the cache so the next call starts as from a fresh engine
-            self.cache.k.zero_()
-            self.cache.v.zero_()
+            self.cache.clear()
             raise
         finally:
             if rng_saved is not None:
@@ -357,7 +356,10 @@ def get_engine(model, batch_size: int, max_length: int) -> DecodeEngine:
     if eng is not None:
         _ENGINES.move_to_end(key)
         return eng
-    need = model.config.num_hidden_layers * 2 * batch_size * model.n_kv_heads * max_length * model.head_dim * 2
+    if hasattr(model, "cache_nbytes"):  # layer-list models: per-layer geometry, recurrent state
+        need = model.cache_nbytes(batch_size, max_length)
+    else:
+        need = model.config.num_hidden_layers * 2 * batch_size * model.n_kv_heads * max_length * model.head_dim * 2
     budget = _engine_budget(model)
     held = sum(e.cache.nbytes() for e in _ENGINES.values())
     while _ENGINES and held + need > budget:
@@ -386,6 +388,8 @@ def generate(model, input_ids, attention_mask=None, generation_config: Optional[
         gc.pad_token_id = model.config.pad_token_id if model.config.pad_token_id >= 0 else 0
     if gc.eos_token_id is None:
         gc.eos_token_id = model.config.eos_token_id
+    if gc.eos_token_id is None:
+        gc.eos_token_id = -1  # no end token: generation runs to max_length
     if prng_key is not None:
         gc.seed = int(prng_key) if not torch.is_tensor(prng_key) else int(prng_key.reshape(-1)[0])
     if s >= gc.max_length:
