@@ -76,7 +76,12 @@ def main():
     ap.add_argument("--mp1-batch", type=int, default=256)
     ap.add_argument("--no-calibration", action="store_true")
     ap.add_argument("--json-out", default=None)
+    ap.add_argument("--hybrid-compare", action="store_true", help="instead of the headline workload: prefill / decode "
+                    "throughput of the Zavevik family beside LLaMA at equal layer sizes (one GPU)")
+    ap.add_argument("--hybrid-sizes", nargs="*", default=["2k", "4k"])
     args = ap.parse_args()
+    if args.hybrid_compare:
+        return _hybrid_compare(args)
 
     import torch
     import torch.distributed as dist
@@ -264,6 +269,15 @@ def main():
     if world > 1:
         dist.barrier()
         dist.destroy_process_group()
+
+
+def _hybrid_compare(args):
+    """``--hybrid-compare``: one JSON line, Zavevik beside LLaMA at equal layer sizes (runtime/benchmark.py)."""
+    import torch
+    from jax_llama_amd.runtime.benchmark import hybrid_compare
+    res = {"metric": "hybrid_family_compare", "n_gpus": 1}
+    res.update(hybrid_compare(torch.device("cuda:0"), sizes=args.hybrid_sizes, progress=_progress))
+    _emit(res, args.json_out)
 
 
 def _box_rooflines(res):

@@ -195,11 +195,175 @@ __global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
   }
 }
 
+// ---- MFMA flash prefill (bf16 caches) ----------------------------------------------------------------------------------
+// One wave = 32 queries of one head, no LDS and no barriers. Keys go by in tiles of 32:
+//   S^T = K Q^T on v_mfma_f32_32x32x16_bf16 with the QUERY on the lane (lane l: query l & 31; its 16 accumulators are 16
+//   of the tile's keys, the other half-wave holds the other 16), so scale, soft cap, bias, mask and the online softmax
+//   are lane-local plus one exchange with lane ^ 32. The key rows are fed in an order (bits 2 and 3 of the row index
+//   swapped) that leaves a lane's accumulators 8c .. 8c + 7 holding keys 16c + 8 (l >> 5) + 0..7: exactly the k-slots
+//   of the B operand of O^T += V^T P^T, so P is used in place. V^T comes from a transposed bf16 copy of the values
+//   (attn_vt_kernel, zero past the last key), 16-byte loads along the keys.
+//   The softmax weights stay 32-bit: P is split into a bf16 high part and a bf16 remainder, two MFMAs per value tile.
+//   Scores of the fast path use exp-based tanh and v_exp_f32; the fp32 format keeps the exact kernel above.
+constexpr int AM_Q = 32, AM_K = 32;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+
+// Vt[b][g][c][j] = V[b][g][j][c] for j < n = *slot + S (0 for n <= j < round_up(n, 32)); grid (Tp / 32, vdim / 32, B * G)
+__global__ void __launch_bounds__(256) attn_vt_kernel(const bf16_t* __restrict__ vc, bf16_t* __restrict__ vt,
+                                                      const int32_t* slot, int S, int T, int Tp, int vdim) {
+  __shared__ bf16_t tile[32][34];
+  const int n = min(*slot + S, T);
+  const int j0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+  if (j0 >= n) return;
+  const size_t bg = blockIdx.z;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  for (int r = ty; r < 32; r += 8) {
+    const int j = j0 + r;
+    tile[r][tx] = j < n ? vc[(bg * T + j) * vdim + c0 + tx] : (bf16_t)0;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) vt[(bg * vdim + c0 + r) * Tp + j0 + tx] = tile[tx][r];
+}
+
+JLA_DEV float am_tanh(float x) {  // 1 - 2 / (e^(2x) + 1), saturating cleanly for large |x|
+  const float e = __expf(2.f * x);
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
+template <int DK, int VT>  // dim = 16 DK, vdim = 32 VT
+__global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf16_t* __restrict__ vt, int Tp) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ql = lane & 31, hi = lane >> 5;
+  const int qblk = (gridDim.x - 1 - blockIdx.x) * 4 + wave;  // long rows first
+  const int s0 = qblk * AM_Q;
+  if (s0 >= p.S) return;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int g = h / (p.H / p.G);
+  const int slot = *p.slot;
+  const int q0 = slot + s0;                 // cache slot of this wave's first query
+  const int sq = min(s0 + ql, p.S - 1);     // (surplus lanes repeat the last query; never stored)
+  const int qi = slot + sq;
+  constexpr int dim = 16 * DK, vdim = 32 * VT;
+  // Q as the B operand: query ql, k-slots 16 kk + 8 hi + e
+  bf16x8_t qf[DK];
+  {
+    const float* q = p.q + (((size_t)b * p.S + sq) * p.H + h) * dim + 8 * hi;
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk) {
+      float f[8];
+      hy_load8(q + 16 * kk, 8, f);
+      qf[kk] = __builtin_bit_cast(bf16x8_t, pack8(f));
+    }
+  }
+  const bf16_t* kbase = reinterpret_cast<const bf16_t*>(p.kc) + ((size_t)b * p.G + g) * p.T * dim;
+  const bf16_t* vbase = vt + ((size_t)b * p.G + g) * vdim * Tp;
+  const int krow = (ql & 0x13) | ((ql & 4) << 1) | ((ql & 8) >> 1);  // bits 2 and 3 swapped
+  f32x16 o[VT];
+#pragma unroll
+  for (int v = 0; v < VT; ++v)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[v][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const int q_last = min(q0 + AM_Q - 1, slot + p.S - 1);
+  const float inv_cap = p.softcap > 0.f ? 1.f / p.softcap : 0.f;
+  for (int j0 = 0; j0 <= q_last; j0 += AM_K) {
+    // scores: rows = keys (fed permuted), columns = queries
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    const bf16_t* kr = kbase + (size_t)min(j0 + krow, p.T - 1) * dim + 8 * hi;
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk) {
+      const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kr + 16 * kk));
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sacc, 0, 0, 0);
+    }
+    // bias of this tile's 63 distances, one per lane: lane t holds distance q0 - j0 - 31 + t
+    float bl = 0.f;
+    const int dbase = q0 - j0 - (AM_K - 1);
+    const bool far = p.bias && dbase >= p.nbias - 1;
+    if (p.bias) bl = p.bias[(size_t)min(max(dbase + lane, 0), p.nbias - 1) * p.H + h];
+    const bool diag = j0 + AM_K - 1 > q0;  // some (query, key) of the tile is masked
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kl = 16 * (r >> 3) + 8 * hi + (r & 7);  // key of accumulator r within the tile
+      float sc = sacc[r] * p.scale;
+      if (p.softcap > 0.f) sc = p.softcap * am_tanh(sc * inv_cap);
+      if (p.bias) sc += far ? bl : __shfl(bl, ql - kl + (AM_K - 1), 64);
+      if (diag && j0 + kl > qi) sc = -INFINITY;
+      sacc[r] = sc;
+      tmax = fmaxf(tmax, sc);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float corr = __expf(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sacc[r] = __expf(sacc[r] - m_new);
+      psum += sacc[r];
+    }
+    l_run = l_run * corr + psum;  // (this half-wave's keys; the halves are added at the end)
+#pragma unroll
+    for (int v = 0; v < VT; ++v)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[v][r] *= corr;
+    // O^T += V^T P^T, P = high bf16 part + bf16 remainder
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      float ph[8], pl[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ph[e] = bf2f(f2bf(sacc[8 * c + e]));
+        pl[e] = sacc[8 * c + e] - ph[e];
+      }
+      const bf16x8_t bh = __builtin_bit_cast(bf16x8_t, pack8(ph)), bo = __builtin_bit_cast(bf16x8_t, pack8(pl));
+#pragma unroll
+      for (int v = 0; v < VT; ++v) {
+        const bf16x8_t vf = __builtin_bit_cast(
+            bf16x8_t, *reinterpret_cast<const u32x4*>(vbase + (size_t)(32 * v + ql) * Tp + j0 + 16 * c + 8 * hi));
+        o[v] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bh, o[v], 0, 0, 0);
+        o[v] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bo, o[v], 0, 0, 0);
+      }
+    }
+  }
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (s0 + ql >= p.S) return;
+  const float inv = 1.f / l_run;
+  float* out = p.out + ((size_t)b * p.S + s0 + ql) * (p.H * vdim) + (size_t)h * vdim;
+#pragma unroll
+  for (int v = 0; v < VT; ++v)
+#pragma unroll
+    for (int r = 0; r < 16; r += 4) {  // rows (value columns) (r & 3) + 8 (r >> 2) + 4 hi: runs of four
+      const float4 w = {o[v][r] * inv, o[v][r + 1] * inv, o[v][r + 2] * inv, o[v][r + 3] * inv};
+      *reinterpret_cast<float4*>(out + 32 * v + 8 * (r >> 2) + 4 * hi) = w;
+    }
+}
+
+template <int DK, int VT>
+static int am_launch(const AttnBias& p, bf16_t* vt, int Tp, hipStream_t s) {
+  attn_vt_kernel<<<dim3(Tp / 32, p.vdim / 32, p.B * p.G), 256, 0, s>>>(reinterpret_cast<const bf16_t*>(p.vc), vt, p.slot,
+                                                                     p.S, p.T, Tp, p.vdim);
+  JLA_CHECK_LAUNCH();
+  attn_bias_mma_kernel<DK, VT><<<dim3((p.S + 127) / 128, p.H, p.B), 256, 0, s>>>(p, vt, Tp);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
+// bytes of the transposed-value workspace the MFMA prefill needs, 0 when the shape goes to the plain kernel
+long long hy_attn_prefill_ws_bytes(int B, int S, int G, int dim, int vdim, int T, int cbf16) {
+  if (!cbf16 || S < 2) return 0;
+  if (!((dim == 64 || dim == 128) && (vdim == 64 || vdim == 128))) return 0;
+  if ((long long)B * G > 65535) return 0;
+  return (long long)B * G * vdim * ((T + 31) / 32 * 32) * 2;
+}
+
 int hy_attn_decode_splits(int B, int H, int t_cap) {
-  // enough waves for the chip (256 CUs x 4 SIMDs), at least 256 keys per split
+  // enough waves for the chip (256 CUs x 4 SIMDs x 2), at least one 64-key step per split
   const long long pairs = (long long)B * H;
   long long want = (2048 + pairs - 1) / (pairs > 0 ? pairs : 1);
-  const long long by_len = (t_cap + 255) / 256;
+  const long long by_len = (t_cap + 63) / 64;
   if (want > by_len) want = by_len;
   if (want < 1) want = 1;
   if (want > 64) want = 64;
@@ -221,6 +385,14 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
     attn_bias_merge_kernel<<<dim3(p.H, p.B), 64, 0, s>>>(p);
     JLA_CHECK_LAUNCH();
     return 0;
+  }
+  if (p.vt_ws && hy_attn_prefill_ws_bytes(p.B, p.S, p.G, p.dim, p.vdim, p.T, p.cbf16) > 0) {
+    const int Tp = (p.T + 31) / 32 * 32;
+    bf16_t* vt = reinterpret_cast<bf16_t*>(p.vt_ws);
+    if (p.dim == 64 && p.vdim == 64) return am_launch<4, 2>(p, vt, Tp, s);
+    if (p.dim == 64 && p.vdim == 128) return am_launch<4, 4>(p, vt, Tp, s);
+    if (p.dim == 128 && p.vdim == 64) return am_launch<8, 2>(p, vt, Tp, s);
+    return am_launch<8, 4>(p, vt, Tp, s);
   }
   dim3 grid((p.S + 3) / 4, p.H, p.B);
   if (p.cbf16) attn_bias_prefill_kernel<bf16_t><<<grid, 256, 0, s>>>(p);

@@ -162,8 +162,12 @@ void attn_prep(Tensor proj, Tensor positions, Tensor slot, int64_t B, int64_t S,
 
 int64_t attn_decode_splits(int64_t B, int64_t H, int64_t t_cap) { return jla::hy_attn_decode_splits(B, H, t_cap); }
 
+int64_t attn_prefill_ws_bytes(int64_t B, int64_t S, int64_t G, int64_t dim, int64_t vdim, int64_t T, bool cbf16) {
+  return jla::hy_attn_prefill_ws_bytes(B, S, G, dim, vdim, T, cbf16);
+}
+
 void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double softcap, OptT bias, Tensor out,
-               int64_t t_cap, OptT ws, int64_t splits) {
+               int64_t t_cap, OptT ws, int64_t splits, OptT vt_ws) {
   jla::AttnBias p{};
   check(q.dim() == 4, "attn_bias: q is [B, S, H, dim]");
   p.B = q.size(0); p.S = q.size(1); p.H = q.size(2); p.dim = q.size(3);
@@ -192,6 +196,13 @@ void attn_bias(Tensor q, Tensor kc, Tensor vc, Tensor slot, double scale, double
     check(ws.has_value() && splits >= 1 && ws->numel() >= (int64_t)p.B * p.H * splits * (p.vdim + 2),
           "attn_bias: decode workspace");
     p.ws = f32w(*ws, "ws");
+  }
+  if (vt_ws.has_value()) {
+    gpu(*vt_ws, "vt_ws");
+    check((int64_t)(vt_ws->numel() * vt_ws->element_size()) >=
+              jla::hy_attn_prefill_ws_bytes(p.B, p.S, p.G, p.dim, p.vdim, p.T, p.cbf16),
+          "attn_bias: transposed-value workspace too small");
+    p.vt_ws = vt_ws->data_ptr();
   }
   rc(jla::hy_attn_bias(p, stream()), "attn_bias");
 }
@@ -276,6 +287,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("attn_prep", &attn_prep);
   m.def("attn_decode_splits", &attn_decode_splits);
   m.def("attn_bias", &attn_bias);
+  m.def("attn_prefill_ws_bytes", &attn_prefill_ws_bytes);
   m.def("delta_prep", &delta_prep);
   m.def("conv_state_update", &conv_state_update);
   m.def("delta_scan", &delta_scan);

@@ -85,8 +85,10 @@ struct AttnBias {
   int t_cap;   // keys the launch may have to cover (decode split sizing); <= T
   float* ws;   // decode split partials: B * H * splits * (vdim + 2) floats
   int splits;
+  void* vt_ws;  // prefill: hy_attn_prefill_ws_bytes(...) bytes for the transposed values (nullptr: the plain kernel)
 };
 int hy_attn_bias(const AttnBias& p, hipStream_t s);
+long long hy_attn_prefill_ws_bytes(int B, int S, int G, int dim, int vdim, int T, int cbf16);
 int hy_attn_decode_splits(int B, int H, int t_cap);
 
 struct DeltaPrep {

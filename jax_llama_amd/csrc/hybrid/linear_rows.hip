@@ -6,7 +6,7 @@
 //  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS. With an
 //    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
 //    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
-//  * few rows (decode): one wave per output column streams the weight row once and dots it with up to 8 rows.
+//  * few rows (decode): a wave streams four weight rows once and dots them with up to 8 activation rows.
 //  * swiglu epilogue: the gate and the up rows of a column are accumulated side by side, out = silu(g) * u.
 // The table router's counting sort is here too.
 #include "hy_util.h"
@@ -138,43 +138,59 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
 JLA_DEV float lr_round(float v, const bf16_t*) { return bf2f(f2bf(v)); }
 JLA_DEV float lr_round(float v, const float*) { return v; }
 
-// One wave per output column; rows [g * MAXR, ...) of group g = blockIdx.y (row_expert: one row per group).
+// A wave owns LR_CPW consecutive output columns: their weight rows are streamed once (16-byte loads, LR_CPW rows in
+// flight per lane) and dotted with the rows [g * rows_per_group, ...) of group g = blockIdx.y (row_expert: one row per
+// group, its expert's weights).
+constexpr int LR_CPW = 4;
+
 template <typename WT, int SWIGLU>
 __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int rows_per_group) {
   constexpr int MAXR = HY_GEMV_MAX_R;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = blockIdx.x * (LR_THREADS / 64) + wave;
-  if (n >= p.N) return;
+  const int n0 = (blockIdx.x * (LR_THREADS / 64) + wave) * LR_CPW;
+  if (n0 >= p.N) return;
   const int r0 = blockIdx.y * rows_per_group;
   const int nr = min(rows_per_group, p.R - r0);
   if (nr <= 0) return;
   const int e = p.row_expert ? p.row_expert[r0] : 0;
   const int K = p.K;
-  const WT* w = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride + (size_t)n * K;
-  const WT* w2 = w + (size_t)p.N * K;
+  const WT* wbase = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride;
+  const WT* w[LR_CPW];
+#pragma unroll
+  for (int c = 0; c < LR_CPW; ++c) w[c] = wbase + (size_t)min(n0 + c, p.N - 1) * K;  // (surplus columns re-read the last)
+  const size_t up = (size_t)p.N * K;
   const float* a[MAXR];
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
     const int rr = r0 + min(r, nr - 1);
     a[r] = p.a + (size_t)(p.a_idx ? p.a_idx[rr] : rr) * p.lda;
   }
-  float acc[MAXR], acc2[MAXR];
+  float acc[MAXR][LR_CPW], acc2[MAXR][LR_CPW];
 #pragma unroll
-  for (int r = 0; r < MAXR; ++r) acc[r] = acc2[r] = 0.f;
+  for (int r = 0; r < MAXR; ++r)
+#pragma unroll
+    for (int c = 0; c < LR_CPW; ++c) acc[r][c] = acc2[r][c] = 0.f;
   for (int k = lane * 8; k < K; k += 64 * 8) {
     const int left = K - k;
-    float wf[8], uf[8], xf[8];
-    hy_load8(w + k, left, wf);
-    if (SWIGLU) hy_load8(w2 + k, left, uf);
+    float wf[LR_CPW][8], uf[LR_CPW][8];
+#pragma unroll
+    for (int c = 0; c < LR_CPW; ++c) {
+      hy_load8(w[c] + k, left, wf[c]);
+      if (SWIGLU) hy_load8(w[c] + up + k, left, uf[c]);
+    }
 #pragma unroll
     for (int r = 0; r < MAXR; ++r) {
       if (r < nr) {
+        float xf[8];
         hy_load8(a[r] + k, left, xf);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const float xv = lr_round(xf[i], w);
-          acc[r] = fmaf(xv, wf[i], acc[r]);
-          if (SWIGLU) acc2[r] = fmaf(xv, uf[i], acc2[r]);
+          const float xv = lr_round(xf[i], wbase);
+#pragma unroll
+          for (int c = 0; c < LR_CPW; ++c) {
+            acc[r][c] = fmaf(xv, wf[c][i], acc[r][c]);
+            if (SWIGLU) acc2[r][c] = fmaf(xv, uf[c][i], acc2[r][c]);
+          }
         }
       }
     }
@@ -182,11 +198,12 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
     if (r < nr) {  // (wave-uniform)
-      const float g = wave_sum(acc[r]);
-      const float u = SWIGLU ? wave_sum(acc2[r]) : 0.f;
-      if (lane == 0) {
-        const int row = r0 + r, drow = p.dst_idx ? p.dst_idx[row] : row;
-        p.out[(size_t)drow * p.ldo + n] = SWIGLU ? hy_silu(g) * u : g;
+      const int row = r0 + r, drow = p.dst_idx ? p.dst_idx[row] : row;
+#pragma unroll
+      for (int c = 0; c < LR_CPW; ++c) {
+        const float g = wave_sum(acc[r][c]);
+        const float u = SWIGLU ? wave_sum(acc2[r][c]) : 0.f;
+        if (lane == 0 && n0 + c < p.N) p.out[(size_t)drow * p.ldo + n0 + c] = SWIGLU ? hy_silu(g) * u : g;
       }
     }
   }
@@ -199,7 +216,7 @@ int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   const bool small = p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert);
   if (small) {
     const int rpg = p.row_expert ? 1 : HY_GEMV_MAX_R;
-    dim3 grid((p.N + 3) / 4, (p.R + rpg - 1) / rpg);
+    dim3 grid((p.N + 4 * LR_CPW - 1) / (4 * LR_CPW), (p.R + rpg - 1) / rpg);
     RowLinear q = p;
     q.offs = nullptr;
     if (p.wbf16) {

@@ -18,6 +18,7 @@ from __future__ import annotations
 
 import importlib
 import math
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -27,6 +28,8 @@ F32 = torch.float32
 
 _EXT = None
 _ERR: Optional[BaseException] = None
+# bf16 prefill attention on the MFMA flash kernel where its shapes apply (JLA_HY_MMA_PREFILL=0: the plain kernel, A/B)
+MMA_PREFILL = os.environ.get("JLA_HY_MMA_PREFILL", "1") != "0"
 
 
 def ext():
@@ -247,12 +250,16 @@ def attn_bias(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slot, scale: 
     out = torch.empty(b * s, h * vdim, dtype=F32, device=q.device)
     e = ext()
     t_cap = int(max_kv) if max_kv is not None else kc.shape[2]
-    ws, splits = None, 1
+    ws, splits, vt = None, 1, None
     if s == 1:
         splits = int(e.attn_decode_splits(b, h, t_cap))
         ws = torch.empty(b * h * splits * (vdim + 2), dtype=F32, device=q.device)
+    elif MMA_PREFILL:
+        nb = int(e.attn_prefill_ws_bytes(b, s, g, dim, vdim, kc.shape[2], kc.dtype == BF16))
+        if nb:  # bf16 caches at the MFMA shapes: the flash kernel over a transposed copy of the values
+            vt = torch.empty(nb // 2, dtype=BF16, device=q.device)
     e.attn_bias(q.contiguous(), kc, vc, _slot_tensor(slot, q.device), float(scale), float(softcap or 0.0), bias, out,
-                t_cap, ws, splits)
+                t_cap, ws, splits, vt)
     return out
 
 

@@ -216,3 +216,68 @@ def calibration(device) -> Dict[str, object]:
 
 def ext_prefetch(e, t: torch.Tensor, grid: int) -> None:
     e.prefetch(t, int(grid))
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Hybrid (Zavevik) family beside LLaMA at equal layer sizes
+# ---------------------------------------------------------------------------------------------------------------
+HYBRID_SIZES = {
+    # name: width, heads, kv heads, head dim, dense FFN width (= the experts' active width), layers, vocab
+    "2k": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ffn=5632, layers=4, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, layers=4, vocab=32000),
+}
+
+
+def zavevik_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int, layers: int, vocab: int,
+                 experts: int = 8, top: int = 2):
+    """A Zavevik config whose layers have a LLaMA layer's sizes: delta, attention, attention on the previous layer's
+    keys, delta, ...; ``experts`` experts of width ``ffn / top`` (the active width equals the dense FFN's)."""
+    from ..config import ZavevikConfig
+    att = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5, softcap=50.0,
+               bias_max=4096, q_temp={"coef": 0.1, "every": 256})
+    dl = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, conv=4)
+    mlp = {"kind": "moe", "expert": {"ff": ffn // top}, "router": {"experts": experts, "top": top}}
+    ls = []
+    for i in range(layers):
+        if i % 4 in (0, 3):
+            ls.append({"type": "delta", "mixer": dict(dl), "mlp": mlp})
+        elif i % 4 == 1:
+            ls.append({"type": "attention", "mixer": dict(att), "mlp": mlp})
+        else:
+            ls.append({"type": "attention", "mixer": dict(att, kv_from=i - 1), "mlp": mlp})
+    return ZavevikConfig.from_dict({"architecture": "Zavevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "token_side": {"dim": 64}, "layers": ls})
+
+
+def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: int = 64, batches=(1, 8),
+                   progress=lambda m: None) -> Dict[str, object]:
+    """Prefill and decode throughput of Zavevik beside LLaMA at equal layer sizes (random weights, bf16, synthetic
+    ids), both through the decode engine: ``prefill_tokens_per_sec`` of one warm ``prompt_len``-token prompt per row
+    and hipGraph-replayed ``decode_ms_per_token`` over ``gen_len`` steps behind it."""
+    from ..config import LLaMAConfig
+    from ..models.llama import LLaMAForCausalLM
+    from ..models.zavevik import ZavevikForCausalLM
+    out: Dict[str, object] = {"prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
+                              "data": "synthetic token ids, random-init weights"}
+    for name in sizes:
+        sz = HYBRID_SIZES[name]
+        row: Dict[str, object] = {"size": sz}
+        for family in ("zavevik", "llama"):
+            if family == "zavevik":
+                model = ZavevikForCausalLM(zavevik_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
+            else:
+                cfg = LLaMAConfig(vocab_size=sz["vocab"], hidden_size=sz["width"], intermediate_size=sz["ffn"],
+                                  num_hidden_layers=sz["layers"], num_attention_heads=sz["heads"],
+                                  num_key_value_heads=sz["kv_heads"], max_sequence_length=prompt_len + gen_len)
+                model = LLaMAForCausalLM(cfg, device=device, _do_init=False).init_random(seed=1)
+            pts = []
+            for b in batches:
+                r = decode_latency(model, b, prompt_len=prompt_len, gen_len=gen_len)
+                r["prefill_tokens_per_sec"] = round(b * prompt_len * 1000.0 / r["prefill_ms"], 1)
+                pts.append(r)
+                progress(f"{name} {family} B={b}: prefill {r['prefill_ms']} ms, decode {r['decode_ms_per_token']} ms")
+            row[family] = {"weight_gb": round(model.weight_bytes() / 1e9, 3), "points": pts}
+            del model
+            torch.cuda.empty_cache()
+        out[name] = row
+    return out
