@@ -79,6 +79,8 @@ def main():
     ap.add_argument("--hybrid-compare", action="store_true", help="instead of the headline workload: prefill / decode "
                     "throughput of the Zavevik family beside LLaMA at equal layer sizes (one GPU)")
     ap.add_argument("--hybrid-sizes", nargs="*", default=["2k", "4k"])
+    ap.add_argument("--hybrid-families", nargs="*", default=["zavevik", "llama"])
+    ap.add_argument("--hybrid-batches", type=int, nargs="*", default=[1, 8])
     args = ap.parse_args()
     if args.hybrid_compare:
         return _hybrid_compare(args)
@@ -276,7 +278,8 @@ def _hybrid_compare(args):
     import torch
     from jax_llama_amd.runtime.benchmark import hybrid_compare
     res = {"metric": "hybrid_family_compare", "n_gpus": 1}
-    res.update(hybrid_compare(torch.device("cuda:0"), sizes=args.hybrid_sizes, progress=_progress))
+    res.update(hybrid_compare(torch.device("cuda:0"), sizes=args.hybrid_sizes, batches=args.hybrid_batches,
+                              families=args.hybrid_families, progress=_progress))
     _emit(res, args.json_out)
 
 

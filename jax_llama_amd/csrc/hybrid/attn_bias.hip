@@ -16,6 +16,11 @@ namespace jla {
 
 JLA_DEV float ab_ld(const float* p) { return *p; }
 JLA_DEV float ab_ld(const bf16_t* p) { return bf2f(*p); }
+JLA_DEV void ab_ld8(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+JLA_DEV void ab_ld8(const bf16_t* p, float* f) { unpack8(*reinterpret_cast<const u32x4*>(p), f); }
 JLA_DEV void ab_st(float* p, float v) { *p = v; }
 JLA_DEV void ab_st(bf16_t* p, float v) { *p = f2bf(v); }
 
@@ -73,31 +78,38 @@ constexpr int AB_MAX_DIM = 512;   // q head held in LDS per wave
 constexpr int AB_MAX_VREG = 8;    // value columns per lane: vdim <= 512
 
 // One wave: keys [j_lo, j_hi) of query (b, h) at slot qi; returns the running max m, sum l and unnormalised acc.
-template <typename CT>
+template <typename CT, int VREG>  // VREG: value columns per lane (vdim <= 64 VREG)
 JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, int j_lo, int j_hi, float& m_run,
                      float& l_run, float* acc) {
+  constexpr int KB = VREG <= 2 ? 16 : 8;  // keys whose value rows are in flight at a time
   const int lane = threadIdx.x & 63;
   const int g = h / (p.H / p.G);
   const CT* kbase = reinterpret_cast<const CT*>(p.kc) + ((size_t)b * p.G + g) * p.T * p.dim;
   const CT* vbase = reinterpret_cast<const CT*>(p.vc) + ((size_t)b * p.G + g) * p.T * p.vdim;
+  const bool fastk = (p.dim & 7) == 0 && ((uintptr_t)kbase & 15) == 0;
   m_run = -INFINITY;
   l_run = 0.f;
 #pragma unroll
-  for (int i = 0; i < AB_MAX_VREG; ++i) acc[i] = 0.f;
+  for (int i = 0; i < VREG; ++i) acc[i] = 0.f;
   for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
     const int j = j0 + lane;
     float sc = -INFINITY;
     if (j < j_hi) {
       const CT* kr = kbase + (size_t)j * p.dim;
       float d0 = 0.f, d1 = 0.f;
-      for (int d = 0; d < p.dim; d += 8) {
-        float kf[8];
-        hy_load8(kr + d, p.dim - d, kf);  // (zeros past dim)
+      if (fastk) {  // whole 16-byte groups: branch-free loads the scheduler can batch
+#pragma unroll 4
+        for (int d = 0; d < p.dim; d += 8) {
+          float kf[8];
+          ab_ld8(kr + d, kf);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-          d0 = fmaf(d + i < p.dim ? qs[d + i] : 0.f, kf[i], d0);
-          d1 = fmaf(d + i + 1 < p.dim ? qs[d + i + 1] : 0.f, kf[i + 1], d1);
+          for (int i = 0; i < 8; i += 2) {
+            d0 = fmaf(qs[d + i], kf[i], d0);
+            d1 = fmaf(qs[d + i + 1], kf[i + 1], d1);
+          }
         }
+      } else {
+        for (int d = 0; d < p.dim; ++d) d0 = fmaf(qs[d], ab_ld(kr + d), d0);
       }
       sc = (d0 + d1) * p.scale;
       if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
@@ -109,22 +121,31 @@ JLA_DEV void ab_wave(const AttnBias& p, const float* qs, int b, int h, int qi, i
     l_run = l_run * corr + wave_sum(pr);
     m_run = m_new;
 #pragma unroll
-    for (int i = 0; i < AB_MAX_VREG; ++i) acc[i] *= corr;
+    for (int i = 0; i < VREG; ++i) acc[i] *= corr;
     const int nk = min(64, j_hi - j0);
-    for (int jj = 0; jj < nk; ++jj) {
-      const float pj = __shfl(pr, jj, 64);
-      const CT* vr = vbase + (size_t)(j0 + jj) * p.vdim;
+    for (int jj = 0; jj < nk; jj += KB) {
+      float vv[KB][VREG];
 #pragma unroll
-      for (int i = 0; i < AB_MAX_VREG; ++i) {
-        const int c = lane + 64 * i;
-        if (c < p.vdim) acc[i] = fmaf(pj, ab_ld(vr + c), acc[i]);
+      for (int u = 0; u < KB; ++u) {
+        const CT* vr = vbase + (size_t)min(j0 + jj + u, j_hi - 1) * p.vdim;
+#pragma unroll
+        for (int i = 0; i < VREG; ++i) {
+          vv[u][i] = ab_ld(vr + min(lane + 64 * i, p.vdim - 1));  // (columns past vdim: never stored)
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < KB; ++u) {
+        const float pj = __shfl(pr, min(jj + u, 63), 64);  // (keys past nk have pr = 0 or repeat a row times 0)
+        const float pw = jj + u < nk ? pj : 0.f;
+#pragma unroll
+        for (int i = 0; i < VREG; ++i) acc[i] = fmaf(pw, vv[u][i], acc[i]);
       }
     }
   }
 }
 
 // prefill: grid (ceil(S / 4), H, B), one wave per query
-template <typename CT>
+template <typename CT, int VREG>
 __global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
   __shared__ float qs_all[4][AB_MAX_DIM];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -135,19 +156,19 @@ __global__ void __launch_bounds__(256) attn_bias_prefill_kernel(AttnBias p) {
   for (int d = lane; d < p.dim; d += 64) qs[d] = q[d];
   __builtin_amdgcn_wave_barrier();
   const int qi = min(*p.slot + s, p.T - 1);
-  float m_run, l_run, acc[AB_MAX_VREG];
-  ab_wave<CT>(p, qs, b, h, qi, 0, qi + 1, m_run, l_run, acc);
+  float m_run, l_run, acc[VREG];
+  ab_wave<CT, VREG>(p, qs, b, h, qi, 0, qi + 1, m_run, l_run, acc);
   float* o = p.out + ((size_t)b * p.S + s) * (p.H * p.vdim) + (size_t)h * p.vdim;
   const float inv = 1.f / l_run;
 #pragma unroll
-  for (int i = 0; i < AB_MAX_VREG; ++i) {
+  for (int i = 0; i < VREG; ++i) {
     const int c = lane + 64 * i;
     if (c < p.vdim) o[c] = acc[i] * inv;
   }
 }
 
 // decode: grid (splits, H, B), one wave per (row, head, split); partial = [m, l, acc[vdim]]
-template <typename CT>
+template <typename CT, int VREG>
 __global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
   __shared__ float qs[AB_MAX_DIM];
   const int lane = threadIdx.x;
@@ -159,39 +180,40 @@ __global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
   const int n = qi + 1;
   const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
   const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
-  float m_run, l_run, acc[AB_MAX_VREG];
-  ab_wave<CT>(p, qs, b, h, qi, j_lo, j_hi, m_run, l_run, acc);
+  float m_run, l_run, acc[VREG];
+  ab_wave<CT, VREG>(p, qs, b, h, qi, j_lo, j_hi, m_run, l_run, acc);
   float* w = p.ws + (((size_t)b * p.H + h) * p.splits + sp) * (p.vdim + 2);
   if (lane == 0) {
     w[0] = m_run;
     w[1] = l_run;
   }
 #pragma unroll
-  for (int i = 0; i < AB_MAX_VREG; ++i) {
+  for (int i = 0; i < VREG; ++i) {
     const int c = lane + 64 * i;
     if (c < p.vdim) w[2 + c] = acc[i];
   }
 }
 
-// grid (H, B), 64 threads: merge the splits in order
+// grid (H, B), 64 threads: merge the splits (at most 64: lane sp holds split sp's maximum and sum)
 __global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
   const int lane = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
   const float* w = p.ws + ((size_t)b * p.H + h) * p.splits * (p.vdim + 2);
-  float m = -INFINITY;
-  for (int sp = 0; sp < p.splits; ++sp) m = fmaxf(m, w[(size_t)sp * (p.vdim + 2)]);
-  float l = 0.f;
-  for (int sp = 0; sp < p.splits; ++sp) {
-    const float* ws = w + (size_t)sp * (p.vdim + 2);
-    if (ws[1] > 0.f) l += ws[1] * expf(ws[0] - m);
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < p.splits) {
+    ms = w[(size_t)lane * (p.vdim + 2)];
+    ls = w[(size_t)lane * (p.vdim + 2) + 1];
   }
+  const float m = wave_max(ls > 0.f ? ms : -INFINITY);
+  const float wt = ls > 0.f ? expf(ms - m) : 0.f;  // weight of this lane's split
+  const float l = wave_sum(ls * wt);
   float* o = p.out + (size_t)b * (p.H * p.vdim) + (size_t)h * p.vdim;
-  for (int c = lane; c < p.vdim; c += 64) {
+  for (int c0 = 0; c0 < p.vdim; c0 += 64) {
+    const int c = min(c0 + lane, p.vdim - 1);
     float a = 0.f;
-    for (int sp = 0; sp < p.splits; ++sp) {
-      const float* ws = w + (size_t)sp * (p.vdim + 2);
-      if (ws[1] > 0.f) a += ws[2 + c] * expf(ws[0] - m);
-    }
-    o[c] = a / l;
+#pragma unroll 8
+    for (int sp = 0; sp < p.splits; ++sp)  // (a split without keys holds zeros and has weight 0)
+      a = fmaf(w[(size_t)sp * (p.vdim + 2) + 2 + c], __shfl(wt, sp, 64), a);
+    if (c0 + lane < p.vdim) o[c] = a / l;
   }
 }
 
@@ -370,6 +392,23 @@ int hy_attn_decode_splits(int B, int H, int t_cap) {
   return (int)want;
 }
 
+// launch KERNEL<cache type, value registers per lane> for p.vdim
+#define AB_BY_VREG(KERNEL, GRID, THREADS)                                              \
+  do {                                                                                 \
+    const int vr = (p.vdim + 63) / 64;                                                 \
+    if (p.cbf16) {                                                                     \
+      if (vr <= 1) KERNEL<bf16_t, 1><<<GRID, THREADS, 0, s>>>(p);                      \
+      else if (vr <= 2) KERNEL<bf16_t, 2><<<GRID, THREADS, 0, s>>>(p);                 \
+      else if (vr <= 4) KERNEL<bf16_t, 4><<<GRID, THREADS, 0, s>>>(p);                 \
+      else KERNEL<bf16_t, 8><<<GRID, THREADS, 0, s>>>(p);                              \
+    } else {                                                                           \
+      if (vr <= 1) KERNEL<float, 1><<<GRID, THREADS, 0, s>>>(p);                       \
+      else if (vr <= 2) KERNEL<float, 2><<<GRID, THREADS, 0, s>>>(p);                  \
+      else if (vr <= 4) KERNEL<float, 4><<<GRID, THREADS, 0, s>>>(p);                  \
+      else KERNEL<float, 8><<<GRID, THREADS, 0, s>>>(p);                               \
+    }                                                                                  \
+  } while (0)
+
 int hy_attn_bias(const AttnBias& p, hipStream_t s) {
   if (p.B < 0 || p.S < 1 || p.H < 1 || p.G < 1 || p.H % p.G || p.T < 1) return -1;
   if (p.dim < 1 || p.dim > AB_MAX_DIM || p.vdim < 1 || p.vdim > 64 * AB_MAX_VREG) return -2;
@@ -379,8 +418,7 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
   if (p.S == 1) {
     if (p.splits < 1 || !p.ws) return -5;
     dim3 grid(p.splits, p.H, p.B);
-    if (p.cbf16) attn_bias_decode_kernel<bf16_t><<<grid, 64, 0, s>>>(p);
-    else attn_bias_decode_kernel<float><<<grid, 64, 0, s>>>(p);
+    AB_BY_VREG(attn_bias_decode_kernel, grid, 64);
     JLA_CHECK_LAUNCH();
     attn_bias_merge_kernel<<<dim3(p.H, p.B), 64, 0, s>>>(p);
     JLA_CHECK_LAUNCH();
@@ -395,8 +433,7 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
     return am_launch<8, 4>(p, vt, Tp, s);
   }
   dim3 grid((p.S + 3) / 4, p.H, p.B);
-  if (p.cbf16) attn_bias_prefill_kernel<bf16_t><<<grid, 256, 0, s>>>(p);
-  else attn_bias_prefill_kernel<float><<<grid, 256, 0, s>>>(p);
+  AB_BY_VREG(attn_bias_prefill_kernel, grid, 256);
   JLA_CHECK_LAUNCH();
   return 0;
 }

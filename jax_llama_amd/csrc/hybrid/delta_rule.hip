@@ -9,9 +9,9 @@
 //                          q and k scaled to unit length (q also by dim^-1/2); beta = sigmoid(.), and the decay
 //                          g = exp(-exp(A_log) softplus(a + dt_bias)).
 //   hy_conv_state_update : the carried tail <- the last taps - 1 inputs of every channel (after hy_delta_prep).
-//   hy_delta_scan        : the recurrence, token by token. A thread owns 32 key rows of one value column in registers;
-//                          the lanes sharing a column (dim / 32 of them, adjacent) combine their partial S^T k and
-//                          S^T q by lane exchange. k, q, v, g, beta of a token are wave-uniform or per-column loads.
+//   hy_delta_scan        : the recurrence, token by token. A thread owns 16 key rows of one value column in registers;
+//                          the lanes sharing a column (dim / 16 of them, adjacent) combine their partial S^T k and
+//                          S^T q by lane exchange. k, q, v, g, beta of the next tokens are staged through LDS.
 //   hy_gated_rmsnorm     : o / rms(o) * w * silu(gate) per head.
 #include "hy_util.h"
 #include "hybrid.h"
@@ -108,44 +108,110 @@ int hy_conv_state_update(const DeltaPrep& p, hipStream_t s) {
   return 0;
 }
 
-constexpr int DS_SLICE = 32;  // key rows per thread
+constexpr int DS_SLICE = 16;    // key rows per thread
+constexpr int DS_STAGE = 4096;  // floats of one staged chunk of tokens (k, q, v, decay, beta) in LDS
+constexpr int DS_PF = DS_STAGE / 256;
 
-// grid (ceil(vdim * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (power of 2)
-__global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
+// Staged element i of the chunk starting at token s0: per token [k (dimp) | q (dimp) | v (cols) | decay | beta | pad],
+// dimp = dim rounded up to the lanes' slices (zeros past dim), cols = the block's value columns [j0, j0 + cols).
+JLA_DEV float ds_src(const DeltaScan& p, int b, int h, int kh, int s0, int j0, int cols, int dimp, int per, int i) {
+  const int t = i / per, e = i - t * per;
+  const size_t m = (size_t)b * p.S + s0 + t;
+  if (e < dimp) return e < p.dim ? p.kn[(m * p.G + kh) * p.dim + e] : 0.f;
+  if (e < 2 * dimp) return e - dimp < p.dim ? p.qn[(m * p.G + kh) * p.dim + (e - dimp)] : 0.f;
+  if (e < 2 * dimp + cols) return p.v[(m * p.H + h) * p.vdim + min(j0 + e - 2 * dimp, p.vdim - 1)];
+  if (e == 2 * dimp + cols) return p.decay[m * p.H + h];
+  if (e == 2 * dimp + cols + 1) return p.beta[m * p.H + h];
+  return 0.f;
+}
+
+// Sum over the R adjacent lanes that share a column (R a power of two); DPP moves up to 16 lanes.
+JLA_DEV float ds_group_sum(float v, int R) {
+  if (R >= 2) v += dppf<0xB1>(v);
+  if (R >= 4) v += dppf<0x4E>(v);
+  if (R >= 8) v += dppf<0x141>(v);
+  if (R >= 16) v += dppf<0x140>(v);
+  if (R >= 32) v += __shfl_xor(v, 16, 64);
+  if (R >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// grid (ceil(vdim * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (power of 2).
+// The tokens' k, q, v, decay and beta are staged ct tokens at a time through LDS (the next chunk's global loads are in
+// flight while the current chunk's steps run), so a step's operands cost LDS latency, not a trip to memory.
+__global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int ct, int per) {
+  __shared__ __attribute__((aligned(16))) float stage[DS_STAGE];
+  const int tid = threadIdx.x;
+  const int t = blockIdx.x * 256 + tid;
   const int h = blockIdx.y, b = blockIdx.z;
   const int j = t / R, r = t - j * R;
   const bool live = j < p.vdim;  // (dead threads still join the lane exchanges)
   const int jc = live ? j : 0;
   const int kh = h / (p.H / p.G);
   const int i0 = r * DS_SLICE;
+  const int j0 = blockIdx.x * (256 / R), cols = 256 / R, jl = j - j0;
+  const int dimp = R * DS_SLICE;
   float S[DS_SLICE];
   float* sp = p.state + (((size_t)b * p.H + h) * p.dim) * p.vdim + jc;
 #pragma unroll
   for (int i = 0; i < DS_SLICE; ++i) S[i] = (live && i0 + i < p.dim) ? sp[(size_t)(i0 + i) * p.vdim] : 0.f;
-  for (int s = 0; s < p.S; ++s) {
-    const size_t m = (size_t)b * p.S + s;
-    const float* k = p.kn + (m * p.G + kh) * p.dim + i0;
-    const float* q = p.qn + (m * p.G + kh) * p.dim + i0;
-    const float g = p.decay[m * p.H + h], beta = p.beta[m * p.H + h];
-    const float v = p.v[(m * p.H + h) * p.vdim + jc];
-    float kv[DS_SLICE], sk = 0.f;
+  float pf[DS_PF];
+  {
+    const int n = min(ct, p.S) * per;  // first chunk
 #pragma unroll
-    for (int i = 0; i < DS_SLICE; ++i) {
-      kv[i] = i0 + i < p.dim ? k[i] : 0.f;
-      S[i] *= g;
-      sk = fmaf(S[i], kv[i], sk);
+    for (int u = 0; u < DS_PF; ++u) {
+      const int i = tid + 256 * u;
+      if (i < n) stage[i] = ds_src(p, b, h, kh, 0, j0, cols, dimp, per, i);
     }
-    for (int o = 1; o < R; o <<= 1) sk += __shfl_xor(sk, o, 64);
-    const float u = beta * (v - sk);
-    float oq = 0.f;
+  }
+  __syncthreads();
+  for (int s0 = 0; s0 < p.S; s0 += ct) {
+    const int nt = min(ct, p.S - s0);
+    const int nn = min(ct, max(p.S - s0 - ct, 0)) * per;  // next chunk's floats
 #pragma unroll
-    for (int i = 0; i < DS_SLICE; ++i) {
-      S[i] = fmaf(kv[i], u, S[i]);
-      oq = fmaf(S[i], i0 + i < p.dim ? q[i] : 0.f, oq);
+    for (int u = 0; u < DS_PF; ++u) {
+      const int i = tid + 256 * u;
+      if (i < nn) pf[u] = ds_src(p, b, h, kh, s0 + ct, j0, cols, dimp, per, i);
     }
-    for (int o = 1; o < R; o <<= 1) oq += __shfl_xor(oq, o, 64);
-    if (live && r == 0) p.o[(m * p.H + h) * p.vdim + j] = oq;
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* row = stage + tt * per;
+      const float4* k4 = reinterpret_cast<const float4*>(row + i0);
+      const float4* q4 = reinterpret_cast<const float4*>(row + dimp + i0);
+      const float v = row[2 * dimp + jl], g = row[2 * dimp + cols], beta = row[2 * dimp + cols + 1];
+      float kv[DS_SLICE], qv[DS_SLICE], sk0 = 0.f, sk1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DS_SLICE; i += 4) {
+        const float4 a = k4[i >> 2], c = q4[i >> 2];
+        kv[i] = a.x; kv[i + 1] = a.y; kv[i + 2] = a.z; kv[i + 3] = a.w;
+        qv[i] = c.x; qv[i + 1] = c.y; qv[i + 2] = c.z; qv[i + 3] = c.w;
+      }
+#pragma unroll
+      for (int i = 0; i < DS_SLICE; i += 2) {
+        S[i] *= g;
+        S[i + 1] *= g;
+        sk0 = fmaf(S[i], kv[i], sk0);
+        sk1 = fmaf(S[i + 1], kv[i + 1], sk1);
+      }
+      const float sk = ds_group_sum(sk0 + sk1, R);
+      const float u = beta * (v - sk);
+      float oq0 = 0.f, oq1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DS_SLICE; i += 2) {
+        S[i] = fmaf(kv[i], u, S[i]);
+        S[i + 1] = fmaf(kv[i + 1], u, S[i + 1]);
+        oq0 = fmaf(S[i], qv[i], oq0);
+        oq1 = fmaf(S[i + 1], qv[i + 1], oq1);
+      }
+      const float oq = ds_group_sum(oq0 + oq1, R);
+      if (live && r == 0) p.o[(((size_t)b * p.S + s0 + tt) * p.H + h) * p.vdim + j] = oq;
+    }
+    __syncthreads();  // every thread is done reading the chunk
+#pragma unroll
+    for (int u = 0; u < DS_PF; ++u) {
+      const int i = tid + 256 * u;
+      if (i < nn) stage[i] = pf[u];
+    }
+    __syncthreads();
   }
 #pragma unroll
   for (int i = 0; i < DS_SLICE; ++i)
@@ -159,8 +225,11 @@ int hy_delta_scan(const DeltaScan& p, hipStream_t s) {
   if (p.H > 65535 || p.B > 65535) return -3;
   int R = 1;
   while (R * DS_SLICE < p.dim) R <<= 1;
+  const int per = (2 * R * DS_SLICE + 256 / R + 2 + 3) / 4 * 4;
+  if (per > DS_STAGE) return -4;
+  const int ct = DS_STAGE / per < 32 ? DS_STAGE / per : 32;
   const long long threads = (long long)p.vdim * R;
-  delta_scan_kernel<<<dim3((unsigned)((threads + 255) / 256), p.H, p.B), 256, 0, s>>>(p, R);
+  delta_scan_kernel<<<dim3((unsigned)((threads + 255) / 256), p.H, p.B), 256, 0, s>>>(p, R, ct, per);
   JLA_CHECK_LAUNCH();
   return 0;
 }

@@ -6,7 +6,7 @@
 //  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS. With an
 //    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
 //    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
-//  * few rows (decode): a wave streams four weight rows once and dots them with up to 8 activation rows.
+//  * few rows (decode): a wave streams one or four weight rows once and dots them with up to 8 activation rows.
 //  * swiglu epilogue: the gate and the up rows of a column are accumulated side by side, out = silu(g) * u.
 // The table router's counting sort is here too.
 #include "hy_util.h"
@@ -138,12 +138,10 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
 JLA_DEV float lr_round(float v, const bf16_t*) { return bf2f(f2bf(v)); }
 JLA_DEV float lr_round(float v, const float*) { return v; }
 
-// A wave owns LR_CPW consecutive output columns: their weight rows are streamed once (16-byte loads, LR_CPW rows in
-// flight per lane) and dotted with the rows [g * rows_per_group, ...) of group g = blockIdx.y (row_expert: one row per
+// A wave owns LR_CPW consecutive output columns (4 for wide outputs such as a vocabulary head, 1 where that would
+// leave too few workgroups): their weight rows are streamed once (16-byte loads, LR_CPW rows in flight per lane) and dotted with the rows [g * rows_per_group, ...) of group g = blockIdx.y (row_expert: one row per
 // group, its expert's weights).
-constexpr int LR_CPW = 4;
-
-template <typename WT, int SWIGLU>
+template <typename WT, int SWIGLU, int LR_CPW>
 __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int rows_per_group) {
   constexpr int MAXR = HY_GEMV_MAX_R;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -170,6 +168,7 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
   for (int r = 0; r < MAXR; ++r)
 #pragma unroll
     for (int c = 0; c < LR_CPW; ++c) acc[r][c] = acc2[r][c] = 0.f;
+#pragma unroll 2
   for (int k = lane * 8; k < K; k += 64 * 8) {
     const int left = K - k;
     float wf[LR_CPW][8], uf[LR_CPW][8];
@@ -216,16 +215,23 @@ int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   const bool small = p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert);
   if (small) {
     const int rpg = p.row_expert ? 1 : HY_GEMV_MAX_R;
-    dim3 grid((p.N + 4 * LR_CPW - 1) / (4 * LR_CPW), (p.R + rpg - 1) / rpg);
+    const int cpw = p.N >= 8192 ? 4 : 1;
+    dim3 grid((p.N + 4 * cpw - 1) / (4 * cpw), (p.R + rpg - 1) / rpg);
     RowLinear q = p;
     q.offs = nullptr;
+#define LR_GEMV(WT, SW)                                                              \
+  do {                                                                               \
+    if (cpw == 4) lr_gemv_kernel<WT, SW, 4><<<grid, LR_THREADS, 0, s>>>(q, rpg);     \
+    else lr_gemv_kernel<WT, SW, 1><<<grid, LR_THREADS, 0, s>>>(q, rpg);              \
+  } while (0)
     if (p.wbf16) {
-      if (p.swiglu) lr_gemv_kernel<bf16_t, 1><<<grid, LR_THREADS, 0, s>>>(q, rpg);
-      else lr_gemv_kernel<bf16_t, 0><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+      if (p.swiglu) LR_GEMV(bf16_t, 1);
+      else LR_GEMV(bf16_t, 0);
     } else {
-      if (p.swiglu) lr_gemv_kernel<float, 1><<<grid, LR_THREADS, 0, s>>>(q, rpg);
-      else lr_gemv_kernel<float, 0><<<grid, LR_THREADS, 0, s>>>(q, rpg);
+      if (p.swiglu) LR_GEMV(float, 1);
+      else LR_GEMV(float, 0);
     }
+#undef LR_GEMV
     JLA_CHECK_LAUNCH();
     return 0;
   }

@@ -250,7 +250,7 @@ def zavevik_like(width: int, heads: int, kv_heads: int, head_dim: int, ffn: int,
 
 
 def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: int = 64, batches=(1, 8),
-                   progress=lambda m: None) -> Dict[str, object]:
+                   families=("zavevik", "llama"), progress=lambda m: None) -> Dict[str, object]:
     """Prefill and decode throughput of Zavevik beside LLaMA at equal layer sizes (random weights, bf16, synthetic
     ids), both through the decode engine: ``prefill_tokens_per_sec`` of one warm ``prompt_len``-token prompt per row
     and hipGraph-replayed ``decode_ms_per_token`` over ``gen_len`` steps behind it."""
@@ -262,7 +262,7 @@ def hybrid_compare(device, sizes=("2k", "4k"), prompt_len: int = 2048, gen_len: 
     for name in sizes:
         sz = HYBRID_SIZES[name]
         row: Dict[str, object] = {"size": sz}
-        for family in ("zavevik", "llama"):
+        for family in families:
             if family == "zavevik":
                 model = ZavevikForCausalLM(zavevik_like(**sz), device=device, dtype=torch.bfloat16, seed=1)
             else:
