@@ -91,7 +91,7 @@ def _scratch_users(remarks: str):
 
 
 # Kernels allowed to use scratch, by mangled-name substring -> max bytes/lane (a rare shape where a spill is accepted).
-# Empty: no kernel of the release or the bounds-checked build spills (re-checked in round 6 after the stream-K, fixup
+# Empty: no kernel of the release or the bounds-checked build spills (re-checked after the stream-K, fixup
 # and exchange-split plans whose epilogue spills these entries used to allow were deleted).
 SCRATCH_OK: dict = {}
 

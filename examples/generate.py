@@ -12,6 +12,11 @@ random-init model of a named architecture with synthetic prompt ids (no checkpoi
   python examples/generate.py --ckpt_dir /ckpt/8B --tokenizer_path /ckpt/tokenizer.model --is_llama3
   torchrun --nproc-per-node 8 --master-addr 127.0.0.1 examples/generate.py --ckpt_dir /ckpt/70B ...
   python examples/generate.py --synthetic --model llama3-8b --max_gen_len 32
+  python examples/generate.py --model_dir /ckpt/zavevik --prompt_ids 5,17,3 --max_gen_len 32 --temperature 0
+
+``--model_dir`` loads any family of the model registry from a directory with ``config.json`` +
+``model.safetensors`` (the family is read from the config) and generates from token ids (such checkpoints
+carry no tokenizer).
 """
 from __future__ import annotations
 
@@ -83,6 +88,20 @@ def synthetic(model_name: str, batch: int, prompt_len: int, max_gen_len: int, te
         print("first row:", seq[0, prompt_len:prompt_len + 16].tolist())
 
 
+def from_model_dir(model_dir: str, prompt_ids: str, max_gen_len: int, temperature: float, top_p: float, dtype: str):
+    """Generate from token ids with a registry model (models/registry.py)."""
+    from jax_llama_amd.models import registry
+    from jax_llama_amd.runtime.engine import GenerationConfig
+    device = "cuda" if torch.cuda.is_available() else "cpu"
+    model = registry.load_model(model_dir, device=device, dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    ids = [int(x) for x in prompt_ids.split(",") if x.strip()]
+    gc = GenerationConfig(max_length=len(ids) + max_gen_len, do_sample=temperature != 0.0, temperature=temperature,
+                          top_p=top_p, pad_token_id=0)
+    seq = model.generate(torch.tensor([ids], dtype=torch.int32), generation_config=gc).sequences[0].tolist()
+    print(registry.architecture_of(model_dir), "generated ids:", seq[len(ids):])
+    return seq
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--ckpt_dir")
@@ -95,8 +114,13 @@ if __name__ == "__main__":
     ap.add_argument("--model", default="llama3-8b")
     ap.add_argument("--batch", type=int, default=2)
     ap.add_argument("--prompt_len", type=int, default=16)
+    ap.add_argument("--model_dir", help="a directory with config.json + model.safetensors of any registered family")
+    ap.add_argument("--prompt_ids", default="1", help="comma-separated prompt token ids (with --model_dir)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     a = ap.parse_args()
-    if a.synthetic:
+    if a.model_dir:
+        from_model_dir(a.model_dir, a.prompt_ids, a.max_gen_len, a.temperature, a.top_p, a.dtype)
+    elif a.synthetic:
         synthetic(a.model, a.batch, a.prompt_len, a.max_gen_len, a.temperature, a.top_p)
     else:
         if not (a.ckpt_dir and a.tokenizer_path):

@@ -3,7 +3,8 @@
 // A is fp32 in memory. With bf16 weights the A tile is rounded to bf16 while it is staged (v_mfma_f32_32x32x16_bf16,
 // fp32 accumulation); with fp32 weights everything stays fp32 on the exact-f32 MFMA (v_mfma_f32_32x32x2_f32).
 //
-//  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS. With an
+//  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS (several
+//    workgroups per CU hide each other's staging; a 128 x 128 tile with register prefetch measured slower). With an
 //    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
 //    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
 //  * few rows (decode): a wave streams one or four weight rows once and dots them with up to 8 activation rows.
@@ -139,19 +140,27 @@ JLA_DEV float lr_round(float v, const bf16_t*) { return bf2f(f2bf(v)); }
 JLA_DEV float lr_round(float v, const float*) { return v; }
 
 // A wave owns LR_CPW consecutive output columns (4 for wide outputs such as a vocabulary head, 1 where that would
-// leave too few workgroups): their weight rows are streamed once (16-byte loads, LR_CPW rows in flight per lane) and dotted with the rows [g * rows_per_group, ...) of group g = blockIdx.y (row_expert: one row per
-// group, its expert's weights).
+// leave too few workgroups): their weight rows are streamed once (16-byte loads, LR_CPW rows in flight per lane) and
+// dotted with the rows of group blockIdx.y: a fixed count of rows, one row with its own expert (row_expert), or every
+// row of one expert of an expert-sorted batch (offs).
 template <typename WT, int SWIGLU, int LR_CPW>
 __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int rows_per_group) {
   constexpr int MAXR = HY_GEMV_MAX_R;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = (blockIdx.x * (LR_THREADS / 64) + wave) * LR_CPW;
   if (n0 >= p.N) return;
-  const int r0 = blockIdx.y * rows_per_group;
-  const int nr = min(rows_per_group, p.R - r0);
-  if (nr <= 0) return;
-  const int e = p.row_expert ? p.row_expert[r0] : 0;
+  // rows of this group: a fixed count, one row with its own expert, or (offs) every row of expert blockIdx.y
+  int g0 = blockIdx.y * rows_per_group, g1 = min(g0 + rows_per_group, p.R), e = 0;
+  if (p.offs) {
+    e = blockIdx.y;
+    g0 = p.offs[e];
+    g1 = p.offs[e + 1];
+  } else if (p.row_expert) {
+    e = p.row_expert[g0];
+  }
   const int K = p.K;
+  for (int r0 = g0; r0 < g1; r0 += MAXR) {  // (more than MAXR rows: the weights are streamed again per 8 rows)
+  const int nr = min(MAXR, g1 - r0);
   const WT* wbase = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride;
   const WT* w[LR_CPW];
 #pragma unroll
@@ -206,19 +215,24 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
       }
     }
   }
+  }
 }
+
+// rows at or below which an expert-sorted batch runs the expert-grouped GEMV (each expert's weights streamed once)
+constexpr int HY_GROUPED_GEMV_MAX_R = 64;
 
 int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   if (p.R < 0 || p.N <= 0 || p.K <= 0 || p.lda < p.K || p.ldo < p.N || p.E < 1) return -1;
   if (p.R == 0) return 0;
   if (p.offs && p.E > 65535) return -2;
-  const bool small = p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert);
+  const bool grouped = p.offs && p.R <= HY_GROUPED_GEMV_MAX_R;
+  const bool small = grouped || (p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert));
   if (small) {
-    const int rpg = p.row_expert ? 1 : HY_GEMV_MAX_R;
+    const int rpg = p.row_expert && !grouped ? 1 : HY_GEMV_MAX_R;
     const int cpw = p.N >= 8192 ? 4 : 1;
-    dim3 grid((p.N + 4 * cpw - 1) / (4 * cpw), (p.R + rpg - 1) / rpg);
+    dim3 grid((p.N + 4 * cpw - 1) / (4 * cpw), grouped ? p.E : (p.R + rpg - 1) / rpg);
     RowLinear q = p;
-    q.offs = nullptr;
+    if (!grouped) q.offs = nullptr;
 #define LR_GEMV(WT, SW)                                                              \
   do {                                                                               \
     if (cpw == 4) lr_gemv_kernel<WT, SW, 4><<<grid, LR_THREADS, 0, s>>>(q, rpg);     \

@@ -13,7 +13,7 @@ experts, expands the distance-bias buckets by distance and keeps the small recur
 
 Number formats: ``dtype=bfloat16`` (serving: bf16 matrix operands and caches, fp32 accumulation, and fp32 residual,
 norms, scores, recurrent state) or ``dtype=float32`` (everything exact fp32). The model runs on the framework's step
-contract -- ``forward_tokens(ids, positions, cache, slot0, ...)`` over an ``init_cache`` object -- so the generation
+interface -- ``forward_tokens(ids, positions, cache, slot0, ...)`` over an ``init_cache`` object -- so the generation
 engine (``runtime/engine.py``) and the request stepper (``runtime/stepper.py``) drive it like LLaMA.
 """
 from __future__ import annotations

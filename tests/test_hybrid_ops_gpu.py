@@ -33,14 +33,14 @@ def test_extension_loaded():
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 7, 24), (3, 64, 320), (8, 130, 72), (9, 4, 320), (70, 392, 320), (200, 96, 24),
-                                   (129, 64, 257)])
+                                   (129, 64, 257), (600, 200, 96), (513, 130, 320)])
 def test_linear(dt, m, n, k):
     x, w = _rand(m, k), _rand(n, k, dt=dt, std=k ** -0.5)
     _close(hy.linear(x.to(DEV), w.to(DEV)), hy.linear(x, w), _tol(dt), "linear")
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("m", [2, 8, 77])
+@pytest.mark.parametrize("m", [2, 8, 77, 530])
 def test_linear_swiglu_strided_rows(dt, m):
     k, n = 96, 40
     big = _rand(m, k + 32)
@@ -50,7 +50,8 @@ def test_linear_swiglu_strided_rows(dt, m):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("m,top,e", [(1, 2, 8), (4, 2, 8), (3, 1, 1), (150, 2, 8), (90, 3, 5), (300, 1, 4)])
+@pytest.mark.parametrize("m,top,e", [(1, 2, 8), (4, 2, 8), (3, 1, 1), (150, 2, 8), (90, 3, 5), (300, 1, 4),
+                                     (20, 2, 8), (21, 3, 2), (9, 1, 1), (700, 2, 3)])
 def test_moe_table(dt, m, top, e):
     d, ff, v = 72, 40, 50
     x = _rand(m, d)

@@ -328,3 +328,39 @@ def test_checkpoint_directory_round_trip(tmp_path):
     ids = torch.tensor([t], dtype=torch.int32)
     assert torch.equal(again(ids).logits, model(ids).logits)
     assert not registry.supports_dtype("llama", F32) and registry.supports_dtype("zavevik", F32)
+
+
+def test_trace_runner_program(tmp_path):
+    """bin/trace_run as a user starts it: steps on standard input, logits files, 'done' lines, rows given back."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    model, sd = build(cfg_full(), "cpu")
+    ckpt, out = str(tmp_path / "ckpt"), str(tmp_path / "out")
+    model.save_pretrained(ckpt, sd)
+    a, b = toks(9, 61, seed=12), toks(5, 61, seed=13)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[6:8], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[8:], "want": [0]}], "end": ["a"]},
+             {"step": 3, "entries": [{"id": "b", "tokens": b, "want": [4]}], "end": ["b"]}]
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", ckpt, "--dtype", "float32",
+                        "--out", out, "--max-tokens", "16", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    assert not os.path.exists(os.path.join(out, "1.f32"))
+    ref_a, _ = oz.forward(cfg_full(), sd, a)
+    ref_b, _ = oz.forward(cfg_full(), sd, b)
+    got0 = np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(2, 61)
+    got2 = np.fromfile(os.path.join(out, "2.f32"), dtype="<f4").reshape(1, 61)
+    got3 = np.fromfile(os.path.join(out, "3.f32"), dtype="<f4").reshape(1, 61)
+    assert err(got0, ref_a[[0, 5]]) < 2e-5 and err(got2, ref_a[[8]]) < 2e-5 and err(got3, ref_b[[4]]) < 2e-5
+    # a family without an all-fp32 path refuses that format at the start
+    llama = tmp_path / "llama"
+    llama.mkdir()
+    (llama / "config.json").write_text(json.dumps({"model_type": "llama"}))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(llama), "--dtype",
+                        "float32", "--out", out, "--device", "cpu"], input="", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 3
