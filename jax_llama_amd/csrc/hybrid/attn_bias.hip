@@ -194,6 +194,87 @@ __global__ void __launch_bounds__(64) attn_bias_decode_kernel(AttnBias p) {
   }
 }
 
+// decode, bf16 caches, dim = 8 DK8 in {64, 128}, vdim = 64 VREG in {64, 128}: the same split as above with every load of
+// a 64-key chunk (the lane's key row, its bias, all 64 value rows) issued before the first use, and q staged into LDS
+// behind them: a decode step is a chain of memory round trips, and this form has two.
+template <int DK8, int VREG>
+__global__ void __launch_bounds__(64) attn_bias_decode_fast_kernel(AttnBias p) {
+  constexpr int dim = 8 * DK8, vdim = 64 * VREG;
+  __shared__ float qs[dim];
+  const int lane = threadIdx.x;
+  const int sp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int g = h / (p.H / p.G);
+  const float* q = p.q + ((size_t)b * p.H + h) * dim;
+  float qv[dim / 64];
+#pragma unroll
+  for (int i = 0; i < dim / 64; ++i) qv[i] = q[lane + 64 * i];
+  const int qi = min(*p.slot, p.T - 1);
+  const int n = qi + 1;
+  const int per = ((n + p.splits - 1) / p.splits + 63) / 64 * 64;
+  const int j_lo = min(n, sp * per), j_hi = min(n, j_lo + per);
+  const bf16_t* kbase = reinterpret_cast<const bf16_t*>(p.kc) + ((size_t)b * p.G + g) * p.T * dim;
+  const bf16_t* vbase = reinterpret_cast<const bf16_t*>(p.vc) + ((size_t)b * p.G + g) * p.T * vdim;
+  float m_run = -INFINITY, l_run = 0.f, acc[VREG];
+#pragma unroll
+  for (int i = 0; i < VREG; ++i) acc[i] = 0.f;
+  bool staged = false;
+  for (int j0 = j_lo; j0 < j_hi; j0 += 64) {
+    const int j = j0 + lane, jc = min(j, j_hi - 1);
+    u32x4 kf[DK8];
+#pragma unroll
+    for (int u = 0; u < DK8; ++u) kf[u] = *reinterpret_cast<const u32x4*>(kbase + (size_t)jc * dim + 8 * u);
+    const float bl = p.bias ? p.bias[(size_t)min(qi - jc, p.nbias - 1) * p.H + h] : 0.f;
+    bf16_t vv[64][VREG];
+#pragma unroll
+    for (int jj = 0; jj < 64; ++jj) {
+      const bf16_t* vr = vbase + (size_t)min(j0 + jj, j_hi - 1) * vdim + lane;
+#pragma unroll
+      for (int i = 0; i < VREG; ++i) vv[jj][i] = vr[64 * i];
+    }
+    if (!staged) {
+#pragma unroll
+      for (int i = 0; i < dim / 64; ++i) qs[lane + 64 * i] = qv[i];
+      __syncthreads();
+      staged = true;
+    }
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int u = 0; u < DK8; ++u) {
+      float f[8];
+      unpack8(kf[u], f);
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        d0 = fmaf(qs[8 * u + i], f[i], d0);
+        d1 = fmaf(qs[8 * u + i + 1], f[i + 1], d1);
+      }
+    }
+    float sc = (d0 + d1) * p.scale;
+    if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
+    sc += bl;
+    if (j >= j_hi) sc = -INFINITY;
+    const float m_new = fmaxf(m_run, wave_max(sc));
+    const float corr = expf(m_run - m_new);
+    const float pr = j < j_hi ? expf(sc - m_new) : 0.f;
+    l_run = l_run * corr + wave_sum(pr);
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < VREG; ++i) acc[i] *= corr;
+#pragma unroll
+    for (int jj = 0; jj < 64; ++jj) {
+      const float pj = __shfl(pr, jj, 64);  // (0 for keys past the split)
+#pragma unroll
+      for (int i = 0; i < VREG; ++i) acc[i] = fmaf(pj, bf2f(vv[jj][i]), acc[i]);
+    }
+  }
+  float* w = p.ws + (((size_t)b * p.H + h) * p.splits + sp) * (vdim + 2);
+  if (lane == 0) {
+    w[0] = m_run;
+    w[1] = l_run;
+  }
+#pragma unroll
+  for (int i = 0; i < VREG; ++i) w[2 + lane + 64 * i] = acc[i];
+}
+
 // grid (H, B), 64 threads: merge the splits (at most 64: lane sp holds split sp's maximum and sum)
 __global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
   const int lane = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
@@ -209,10 +290,15 @@ __global__ void __launch_bounds__(64) attn_bias_merge_kernel(AttnBias p) {
   float* o = p.out + (size_t)b * (p.H * p.vdim) + (size_t)h * p.vdim;
   for (int c0 = 0; c0 < p.vdim; c0 += 64) {
     const int c = min(c0 + lane, p.vdim - 1);
+    float part[64];
+#pragma unroll
+    for (int sp = 0; sp < 64; ++sp) part[sp] = w[(size_t)min(sp, p.splits - 1) * (p.vdim + 2) + 2 + c];  // one round trip
     float a = 0.f;
-#pragma unroll 8
-    for (int sp = 0; sp < p.splits; ++sp)  // (a split without keys holds zeros and has weight 0)
-      a = fmaf(w[(size_t)sp * (p.vdim + 2) + 2 + c], __shfl(wt, sp, 64), a);
+#pragma unroll
+    for (int sp = 0; sp < 64; ++sp) {  // (a split without keys holds zeros and has weight 0)
+      const float ws = __shfl(wt, sp, 64);
+      a = fmaf(part[sp], sp < p.splits ? ws : 0.f, a);
+    }
     if (c0 + lane < p.vdim) o[c] = a / l;
   }
 }
@@ -417,8 +503,16 @@ int hy_attn_bias(const AttnBias& p, hipStream_t s) {
   if (p.H > 65535 || p.B > 65535) return -4;
   if (p.S == 1) {
     if (p.splits < 1 || !p.ws) return -5;
+    if (p.splits > 64) return -6;  // (the merge holds one split per lane)
     dim3 grid(p.splits, p.H, p.B);
-    AB_BY_VREG(attn_bias_decode_kernel, grid, 64);
+    if (p.cbf16 && (p.dim == 64 || p.dim == 128) && (p.vdim == 64 || p.vdim == 128)) {
+      if (p.dim == 64 && p.vdim == 64) attn_bias_decode_fast_kernel<8, 1><<<grid, 64, 0, s>>>(p);
+      else if (p.dim == 64) attn_bias_decode_fast_kernel<8, 2><<<grid, 64, 0, s>>>(p);
+      else if (p.vdim == 64) attn_bias_decode_fast_kernel<16, 1><<<grid, 64, 0, s>>>(p);
+      else attn_bias_decode_fast_kernel<16, 2><<<grid, 64, 0, s>>>(p);
+    } else {
+      AB_BY_VREG(attn_bias_decode_kernel, grid, 64);
+    }
     JLA_CHECK_LAUNCH();
     attn_bias_merge_kernel<<<dim3(p.H, p.B), 64, 0, s>>>(p);
     JLA_CHECK_LAUNCH();

@@ -8,7 +8,8 @@
 //                          inputs before this call come from the carried tail, zeros at a sequence start), SiLU, then
 //                          q and k scaled to unit length (q also by dim^-1/2); beta = sigmoid(.), and the decay
 //                          g = exp(-exp(A_log) softplus(a + dt_bias)).
-//   hy_conv_state_update : the carried tail <- the last taps - 1 inputs of every channel (after hy_delta_prep).
+//   hy_conv_state_update : the carried tail <- the last taps - 1 inputs of every channel (after hy_delta_prep; a
+//                          one-token step does it inside hy_delta_prep and launches nothing here).
 //   hy_delta_scan        : the recurrence, token by token. A thread owns 16 key rows of one value column in registers;
 //                          the lanes sharing a column (dim / 16 of them, adjacent) combine their partial S^T k and
 //                          S^T q by lane exchange. k, q, v, g, beta of the next tokens are staged through LDS.
@@ -57,6 +58,12 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(DeltaPrep p) {
     y = hy_silu(y);
     dst[d] = y;
     ss = fmaf(y, y, ss);
+    if (p.S == 1 && p.taps > 1) {  // one token: this lane is the channel's only reader, so it advances the tail itself
+      const int C = 2 * p.G * p.dim + p.H * p.vdim, n = p.taps - 1;
+      float* st = p.conv_state + ((size_t)b * C + c) * n;
+      for (int i = 0; i + 1 < n; ++i) st[i] = st[i + 1];
+      st[n - 1] = p.proj[(size_t)m * p.ld + c];
+    }
   }
   if (kind == 2) return;
   ss = wave_sum(ss);
@@ -101,7 +108,7 @@ int hy_delta_prep(const DeltaPrep& p, hipStream_t s) {
 
 int hy_conv_state_update(const DeltaPrep& p, hipStream_t s) {
   if (int r = dp_check(p)) return r;
-  if (p.B == 0 || p.taps == 1) return 0;
+  if (p.B == 0 || p.taps == 1 || p.S == 1) return 0;  // (S = 1: hy_delta_prep advanced the tail itself)
   const long long n = (long long)p.B * (2 * p.G * p.dim + p.H * p.vdim);
   conv_state_update_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p);
   JLA_CHECK_LAUNCH();

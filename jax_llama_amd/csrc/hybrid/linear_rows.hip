@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
   for (int r = 0; r < MAXR; ++r)
 #pragma unroll
     for (int c = 0; c < LR_CPW; ++c) acc[r][c] = acc2[r][c] = 0.f;
-#pragma unroll 2
+#pragma unroll 4
   for (int k = lane * 8; k < K; k += 64 * 8) {
     const int left = K - k;
     float wf[LR_CPW][8], uf[LR_CPW][8];

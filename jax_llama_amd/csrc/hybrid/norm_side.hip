@@ -29,12 +29,42 @@ int hy_embed_rows(const int32_t* ids, const void* table, int wbf16, int V, int l
   return 0;
 }
 
-// one workgroup per row
+// one workgroup per row; rows of up to 4096 columns are held in registers (y, x and the gain loaded in one round trip)
+constexpr int NR_REGS = 16;
+
 __global__ void __launch_bounds__(256) norm_residual_kernel(const float* y, int nsum, float ysc, const float* w,
                                                             int w_vec, float eps, float* x, float* out, int D) {
   __shared__ float red[16];
   const int m = blockIdx.x;
   const float* yr = y + (size_t)m * nsum * D;
+  if (D <= 256 * NR_REGS) {
+    float v[NR_REGS], xv[NR_REGS], wv[NR_REGS];
+    const float w0 = w_vec ? 0.f : w[0];
+#pragma unroll
+    for (int u = 0; u < NR_REGS; ++u) {
+      v[u] = xv[u] = wv[u] = 0.f;
+      if (256 * u < D) {  // (uniform)
+        const int d = min(threadIdx.x + 256 * u, D - 1);
+        float a = 0.f;
+        for (int c = 0; c < nsum; ++c) a += yr[(size_t)c * D + d];
+        v[u] = a * ysc;
+        xv[u] = x ? x[(size_t)m * D + d] : 0.f;
+        wv[u] = w_vec ? w[d] : w0;
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NR_REGS; ++u)
+      if (threadIdx.x + 256 * u < D) ss = fmaf(v[u], v[u], ss);
+    ss = block_sum(ss, red);
+    const float sc = 1.f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int u = 0; u < NR_REGS; ++u) {
+      const int d = threadIdx.x + 256 * u;
+      if (d < D) (x ? x : out)[(size_t)m * D + d] = xv[u] + v[u] * sc * wv[u];
+    }
+    return;
+  }
   float ss = 0.f;
   for (int d = threadIdx.x; d < D; d += 256) {
     float v = 0.f;
