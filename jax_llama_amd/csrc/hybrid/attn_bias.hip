@@ -374,17 +374,36 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
   float m_run = -INFINITY, l_run = 0.f;
   const int q_last = min(q0 + AM_Q - 1, slot + p.S - 1);
   const float inv_cap = p.softcap > 0.f ? 1.f / p.softcap : 0.f;
+  // the next tile's key and value fragments are loaded while the current tile is computed (one wave per SIMD at small
+  // batch: nothing else hides the loads)
+  u32x4 kn[DK], vn[2][VT];
+  auto fetch = [&](int j0) {
+    const bf16_t* kr = kbase + (size_t)min(j0 + krow, p.T - 1) * dim + 8 * hi;
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk) kn[kk] = *reinterpret_cast<const u32x4*>(kr + 16 * kk);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int v = 0; v < VT; ++v)
+        vn[c][v] = *reinterpret_cast<const u32x4*>(vbase + (size_t)(32 * v + ql) * Tp + min(j0, Tp - AM_K) + 16 * c + 8 * hi);
+  };
+  fetch(0);
   for (int j0 = 0; j0 <= q_last; j0 += AM_K) {
+    u32x4 kc_[DK], vc_[2][VT];
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk) kc_[kk] = kn[kk];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int v = 0; v < VT; ++v) vc_[c][v] = vn[c][v];
+    fetch(j0 + AM_K);  // (past the last tile: clamped addresses, never used)
     // scores: rows = keys (fed permuted), columns = queries
     f32x16 sacc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-    const bf16_t* kr = kbase + (size_t)min(j0 + krow, p.T - 1) * dim + 8 * hi;
 #pragma unroll
-    for (int kk = 0; kk < DK; ++kk) {
-      const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kr + 16 * kk));
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sacc, 0, 0, 0);
-    }
+    for (int kk = 0; kk < DK; ++kk)
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kc_[kk]), qf[kk], sacc, 0, 0, 0);
     // bias of this tile's 63 distances, one per lane: lane t holds distance q0 - j0 - 31 + t
     float bl = 0.f;
     const int dbase = q0 - j0 - (AM_K - 1);
@@ -429,8 +448,7 @@ __global__ void __launch_bounds__(256) attn_bias_mma_kernel(AttnBias p, const bf
       const bf16x8_t bh = __builtin_bit_cast(bf16x8_t, pack8(ph)), bo = __builtin_bit_cast(bf16x8_t, pack8(pl));
 #pragma unroll
       for (int v = 0; v < VT; ++v) {
-        const bf16x8_t vf = __builtin_bit_cast(
-            bf16x8_t, *reinterpret_cast<const u32x4*>(vbase + (size_t)(32 * v + ql) * Tp + j0 + 16 * c + 8 * hi));
+        const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, vc_[c][v]);
         o[v] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bh, o[v], 0, 0, 0);
         o[v] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, bo, o[v], 0, 0, 0);
       }

@@ -121,6 +121,12 @@ void norm_residual(Tensor y, int64_t nsum, double ysc, Tensor w, double eps, Opt
      "norm_residual");
 }
 
+void cast_bf16(Tensor x, Tensor y) {
+  gpu(y, "y");
+  check(y.scalar_type() == torch::kBFloat16 && y.numel() == x.numel() && x.numel() % 8 == 0, "cast_bf16 shapes");
+  rc(jla::hy_cast_bf16(f32(x, "x"), reinterpret_cast<jla::bf16_t*>(y.data_ptr()), x.numel(), stream()), "cast_bf16");
+}
+
 void gelu_gate_rows(Tensor gp, Tensor ids, Tensor table, int64_t col0, Tensor g) {
   const int wb = wtype(table, "table");
   check(gp.dim() == 2 && table.dim() == 2 && g.sizes() == gp.sizes(), "gelu_gate_rows shapes");
@@ -284,6 +290,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("route_table", &route_table);
   m.def("norm_residual", &norm_residual);
   m.def("gelu_gate_rows", &gelu_gate_rows);
+  m.def("cast_bf16", &cast_bf16);
   m.def("attn_prep", &attn_prep);
   m.def("attn_decode_splits", &attn_decode_splits);
   m.def("attn_bias", &attn_bias);

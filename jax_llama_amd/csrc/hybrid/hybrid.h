@@ -48,6 +48,10 @@ int hy_route_table(const int32_t* ids, const int32_t* table, int V, int M, int t
 int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_vec, float eps, float* x, float* out,
                      int M, int D, hipStream_t s);
 
+// y (bf16) = x (fp32), n a multiple of 8
+typedef uint16_t bf16_t;
+int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s);
+
 // g[m, c] = gelu_tanh(gp[m, c]) * table[ids[m], col0 + c]
 int hy_gelu_gate_rows(const float* gp, const int32_t* ids, const void* table, int wbf16, int V, int ld, int col0,
                       float* g, int M, int D, hipStream_t s);

@@ -4,7 +4,7 @@
 // fp32 accumulation); with fp32 weights everything stays fp32 on the exact-f32 MFMA (v_mfma_f32_32x32x2_f32).
 //
 //  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS (several
-//    workgroups per CU hide each other's staging; a 128 x 128 tile with register prefetch measured slower). With an
+//    workgroups per CU hide each other's staging; a 128 x 128 tile with register prefetch and a 64-deep K stage measured slower). With an
 //    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
 //    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
 //  * few rows (decode): a wave streams one or four weight rows once and dots them with up to 8 activation rows.
@@ -94,27 +94,30 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
   for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += LR_BK) {
-    const int gk = k0 + skq, left = K - gk;
-    float f[8];
-    if (a_ptr && left > 0) hy_load8(a_ptr + gk, left, f);
-    else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) f[i] = 0.f;
-    }
-    lr_store8(&As[srow * LD + skq], f);
-    if (w_ptr && left > 0) hy_load8(w_ptr + gk, left, f);
-    else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) f[i] = 0.f;
-    }
-    lr_store8(&Bs[srow * LD + skq], f);
-    if (SWIGLU) {
-      if (w2_ptr && left > 0) hy_load8(w2_ptr + gk, left, f);
+    for (int half = 0; half < LR_BK / 32; ++half) {  // a thread stages 8 k of its row per 32-wide half
+      const int kq = skq + 32 * half, gk = k0 + kq, left = K - gk;
+      float f[8];
+      if (a_ptr && left > 0) hy_load8(a_ptr + gk, left, f);
       else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) f[i] = 0.f;
       }
-      lr_store8(&Bs[(LR_BN + srow) * LD + skq], f);
+      lr_store8(&As[srow * LD + kq], f);
+      if (w_ptr && left > 0) hy_load8(w_ptr + gk, left, f);
+      else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = 0.f;
+      }
+      lr_store8(&Bs[srow * LD + kq], f);
+      if (SWIGLU) {
+        if (w2_ptr && left > 0) hy_load8(w2_ptr + gk, left, f);
+        else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) f[i] = 0.f;
+        }
+        lr_store8(&Bs[(LR_BN + srow) * LD + kq], f);
+      }
     }
     __syncthreads();
     const WT* a_row = &As[(wm * 32 + (lane & 31)) * LD];

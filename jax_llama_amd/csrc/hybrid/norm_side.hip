@@ -93,6 +93,24 @@ int hy_norm_residual(const float* y, int nsum, float ysc, const float* w, int w_
   return 0;
 }
 
+// bf16 copy of an fp32 activation (the A operand of the packed MFMA GEMMs), 8 elements per thread
+__global__ void __launch_bounds__(256) cast_bf16_kernel(const float* __restrict__ x, bf16_t* __restrict__ y, long long n8) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  float f[8];
+  hy_load8(x + 8 * i, 8, f);
+  *reinterpret_cast<u32x4*>(y + 8 * i) = pack8(f);
+}
+
+int hy_cast_bf16(const float* x, bf16_t* y, long long n, hipStream_t s) {
+  if (n < 0 || n % 8) return -1;
+  if (n == 0) return 0;
+  const long long n8 = n / 8;
+  cast_bf16_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, s>>>(x, y, n8);
+  JLA_CHECK_LAUNCH();
+  return 0;
+}
+
 JLA_DEV float ns_gelu_tanh(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }

@@ -90,6 +90,33 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor, col0: int = 0, ncols: Opt
     return out
 
 
+# Dense bf16 linears of a prompt-sized batch run on the framework's tuned MFMA GEMM (ops.linear over the fragment-
+# packed weight layout, csrc/kernels/gemm.hip) when the main extension is built and the shape fits its layout
+# (N % 16 == 0, K % 32 == 0); the row-major kernel here serves every other case. JLA_HY_PACKED_GEMM=0: never.
+PACKED_GEMM = os.environ.get("JLA_HY_PACKED_GEMM", "1") != "0"
+PACKED_GEMM_MIN_M = 256
+_PACKED = {}
+
+
+def _packed_weight(w: torch.Tensor):
+    """The fragment-packed copy of a dense ``[N, K]`` bf16 weight (made once, kept beside the row-major one)."""
+    key = (w.data_ptr(), tuple(w.shape))
+    pw = _PACKED.get(key)
+    if pw is None or pw[0] is not w:
+        from ..models.weights import PackedLinear
+        pw = _PACKED[key] = (w, PackedLinear.from_dense(w, w.device))
+    return pw[1]
+
+
+def _use_packed_gemm(x: torch.Tensor, w: torch.Tensor) -> bool:
+    if not PACKED_GEMM or w.dtype != BF16 or w.dim() != 2 or x.shape[0] < PACKED_GEMM_MIN_M:
+        return False
+    if w.shape[0] % 16 or w.shape[1] % 32 or not x.is_contiguous():
+        return False
+    from . import ext_available as core_available
+    return core_available()
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
     """``x [M, K] (fp32) @ w [N, K]^T`` -> fp32 ``[M, N]``; ``swiglu``: ``w`` is ``[2N, K]`` (gate rows, then up rows)
     and the result is ``silu(x Wg^T) * (x Wu^T)``. ``x`` may be a column-contiguous view with strided rows."""
@@ -97,6 +124,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False) -> torch.Tens
     if not _gpu(x):
         y = _round_like(x, w) @ w.float().t()
         return torch.nn.functional.silu(y[:, :n]) * y[:, n:] if swiglu else y
+    if not swiglu and _use_packed_gemm(x, w):
+        from . import linear as packed_linear
+        xb = torch.empty(x.shape, dtype=BF16, device=x.device)
+        ext().cast_bf16(x, xb)
+        return packed_linear(xb, _packed_weight(w), out_dtype=F32)
     out = torch.empty(x.shape[0], n, dtype=F32, device=x.device)
     ext().linear_rows(x, None, w, out, None, None, None, x.shape[0], bool(swiglu))
     return out

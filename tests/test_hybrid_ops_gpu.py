@@ -145,3 +145,21 @@ def test_delta_rule(shape):
     gate, w = _rand(b * s, h * vdim), torch.rand(vdim) + 0.5
     _close(hy.gated_rmsnorm(o_ref.to(DEV), gate.to(DEV), w.to(DEV), 1e-6), hy.gated_rmsnorm(o_ref, gate, w, 1e-6), 2e-5,
            "gated norm")
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 64, 96), (777, 400, 320), (2048, 16, 32)])
+def test_linear_on_the_packed_gemm(m, n, k):
+    """Prompt-sized dense bf16 linears go to the framework's fragment-packed MFMA GEMM when the main extension is
+    built; same operands, so the result matches the row-major kernel and the CPU op up to summation order."""
+    from jax_llama_amd import ops
+    x, w = _rand(m, k), _rand(n, k, dt=torch.bfloat16, std=k ** -0.5)
+    xg, wg = x.to(DEV), w.to(DEV)
+    assert hy._use_packed_gemm(xg, wg) == ops.ext_available()
+    got = hy.linear(xg, wg)
+    _close(got, hy.linear(x, w), 2e-5, "packed gemm vs cpu")
+    hy.PACKED_GEMM = False
+    try:
+        _close(hy.linear(xg, wg), got, 2e-5, "row-major kernel vs packed gemm")
+    finally:
+        hy.PACKED_GEMM = True
+    assert not hy._use_packed_gemm(xg[:100], wg) and not hy._use_packed_gemm(xg, wg[:15])
