@@ -254,13 +254,14 @@ class MixerSpec:
     def from_dict(cls, type_: str, d: Dict[str, Any]) -> "MixerSpec":
         d = dict(d)
         qt = d.pop("q_temp", None) or {}
-        known = dict(type=type_, heads=int(d.pop("heads")), kv_heads=int(d.pop("kv_heads")), dim=int(d.pop("dim")),
-                     vdim=int(d.pop("vdim")), conv=int(d.pop("conv", 0)), scale=float(d.pop("scale", 1.0)),
+        heads, dim = int(d.pop("heads")), int(d.pop("dim"))
+        known = dict(type=type_, heads=heads, kv_heads=int(d.pop("kv_heads", heads)), dim=dim,
+                     vdim=int(d.pop("vdim", dim)), conv=int(d.pop("conv", 1 if type_ == "delta" else 0)),
+                     scale=float(d.pop("scale", 1.0)),
                      softcap=float(d.pop("softcap", 0.0) or 0.0), bias_max=int(d.pop("bias_max", 0) or 0),
                      q_temp_coef=float(qt.get("coef", 0.0)), q_temp_every=int(qt.get("every", 1)),
                      kv_from=d.pop("kv_from", None))
-        if d:
-            raise ValueError(f"unknown mixer keys {sorted(d)}")
+        # (keys this family does not define are ignored, like HF configs keep unknown entries)
         if known["kv_from"] is not None:
             known["kv_from"] = int(known["kv_from"])
         if type_ not in ("attention", "delta"):
