@@ -364,3 +364,38 @@ def test_trace_runner_program(tmp_path):
     r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(llama), "--dtype",
                         "float32", "--out", out, "--device", "cpu"], input="", capture_output=True, text=True, timeout=300)
     assert r.returncode == 3
+
+
+def cfg_mfma_shapes():
+    """Head sizes of the MFMA attention kernels (64 / 128), three query heads per key head, six layers in another
+    order, two layers on shared keys, a distance table that reaches a few hundred keys."""
+    a64 = dict(heads=6, kv_heads=2, dim=64, vdim=128, scale=0.125, softcap=30.0, bias_max=300,
+               q_temp={"coef": 0.3, "every": 64})
+    a128 = dict(heads=2, kv_heads=1, dim=128, vdim=64, scale=0.09, bias_max=150)
+    dl = dict(heads=4, kv_heads=2, dim=64, vdim=48, conv=4)
+    return {"architecture": "Zavevik", "vocab": 300, "width": 192, "norm": {"eps": 1e-6}, "token_side": {"dim": 16},
+            "layers": [{"type": "attention", "mixer": dict(a64), "mlp": _moe(4, 2, 96)},
+                       {"type": "attention", "mixer": dict(a64, kv_from=0), "mlp": None},
+                       {"type": "delta", "mixer": dict(dl), "mlp": _moe(4, 2, 96)},
+                       {"type": "attention", "mixer": dict(a128), "mlp": _moe(6, 3, 64)},
+                       {"type": "delta", "mixer": dict(dl, heads=2, kv_heads=1, dim=128, vdim=128), "mlp": None},
+                       {"type": "attention", "mixer": dict(a128, kv_from=3, softcap=5.0), "mlp": _moe(4, 1, 96)}]}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_longer_prompts_at_the_mfma_head_sizes(dtype):
+    """600 tokens in uneven portions (prompt-sized GEMMs, the flash prefill starting at unaligned slots, decode over
+    several key splits) on the GPU against the framework's fp32 CPU path, which the tests above tie to the oracle."""
+    cfg = cfg_mfma_shapes()
+    ref_model, sd = build(cfg, "cpu", F32, buckets=32)
+    t = toks(600, 300, seed=21)
+    with torch.no_grad():
+        ref = ref_model(torch.tensor([t], dtype=torch.int32)).logits[0].numpy()
+    model = ZavevikForCausalLM(ZavevikConfig.from_dict(cfg), device="cuda", dtype=dtype, _do_init=False).load_state_dict(sd)
+    portions = [261, 3, 2, 190, 64, 37] + [1] * 43
+    got = run_portions(model, t, portions)
+    e = [err(got[i], ref[i]) for i in range(600)]
+    assert max(e) < (2e-4 if dtype == F32 else 4e-2), (int(np.argmax(e)), max(e))
+    whole = run_portions(model, t, [600])
+    assert err(whole, got) < (2e-5 if dtype == F32 else 2e-2)
