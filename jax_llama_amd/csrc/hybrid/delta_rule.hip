@@ -116,16 +116,23 @@ int hy_conv_state_update(const DeltaPrep& p, hipStream_t s) {
 }
 
 constexpr int DS_SLICE = 16;    // key rows per thread
+constexpr int DS_PITCH = 20;    // floats between the staged slices of k / q: the lanes' 16-byte reads fall on distinct banks
 constexpr int DS_STAGE = 4096;  // floats of one staged chunk of tokens (k, q, v, decay, beta) in LDS
 constexpr int DS_PF = DS_STAGE / 256;
 
 // Staged element i of the chunk starting at token s0: per token [k (dimp) | q (dimp) | v (cols) | decay | beta | pad],
-// dimp = dim rounded up to the lanes' slices (zeros past dim), cols = the block's value columns [j0, j0 + cols).
-JLA_DEV float ds_src(const DeltaScan& p, int b, int h, int kh, int s0, int j0, int cols, int dimp, int per, int i) {
-  const int t = i / per, e = i - t * per;
+// dimp = R slices of DS_PITCH floats (16 values + 4 pad; zeros past dim), cols = the block's value columns
+// [j0, j0 + cols).
+JLA_DEV float ds_src(const DeltaScan& p, int b, int h, int kh, int s0, int j0, int cols, int dimp, int per,
+                     unsigned per_magic, int i) {
+  const int t = (int)__umulhi((unsigned)i, per_magic), e = i - t * per;  // i / per (exact for i < 2^16)
   const size_t m = (size_t)b * p.S + s0 + t;
-  if (e < dimp) return e < p.dim ? p.kn[(m * p.G + kh) * p.dim + e] : 0.f;
-  if (e < 2 * dimp) return e - dimp < p.dim ? p.qn[(m * p.G + kh) * p.dim + (e - dimp)] : 0.f;
+  if (e < 2 * dimp) {
+    const int ee = e < dimp ? e : e - dimp;
+    const int sl = ee / DS_PITCH, w = ee - sl * DS_PITCH, d = sl * DS_SLICE + w;
+    if (w >= DS_SLICE || d >= p.dim) return 0.f;
+    return (e < dimp ? p.kn : p.qn)[(m * p.G + kh) * p.dim + d];
+  }
   if (e < 2 * dimp + cols) return p.v[(m * p.H + h) * p.vdim + min(j0 + e - 2 * dimp, p.vdim - 1)];
   if (e == 2 * dimp + cols) return p.decay[m * p.H + h];
   if (e == 2 * dimp + cols + 1) return p.beta[m * p.H + h];
@@ -146,7 +153,7 @@ JLA_DEV float ds_group_sum(float v, int R) {
 // grid (ceil(vdim * R / 256), H, B); thread -> (column j = t / R, slice r = t % R), R = lanes per column (power of 2).
 // The tokens' k, q, v, decay and beta are staged ct tokens at a time through LDS (the next chunk's global loads are in
 // flight while the current chunk's steps run), so a step's operands cost LDS latency, not a trip to memory.
-__global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int ct, int per) {
+__global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int ct, int per, unsigned per_magic) {
   __shared__ __attribute__((aligned(16))) float stage[DS_STAGE];
   const int tid = threadIdx.x;
   const int t = blockIdx.x * 256 + tid;
@@ -157,7 +164,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int
   const int kh = h / (p.H / p.G);
   const int i0 = r * DS_SLICE;
   const int j0 = blockIdx.x * (256 / R), cols = 256 / R, jl = j - j0;
-  const int dimp = R * DS_SLICE;
+  const int dimp = R * DS_PITCH;
   float S[DS_SLICE];
   float* sp = p.state + (((size_t)b * p.H + h) * p.dim) * p.vdim + jc;
 #pragma unroll
@@ -168,7 +175,7 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int
 #pragma unroll
     for (int u = 0; u < DS_PF; ++u) {
       const int i = tid + 256 * u;
-      if (i < n) stage[i] = ds_src(p, b, h, kh, 0, j0, cols, dimp, per, i);
+      if (i < n) stage[i] = ds_src(p, b, h, kh, 0, j0, cols, dimp, per, per_magic, i);
     }
   }
   __syncthreads();
@@ -178,12 +185,12 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaScan p, int R, int
 #pragma unroll
     for (int u = 0; u < DS_PF; ++u) {
       const int i = tid + 256 * u;
-      if (i < nn) pf[u] = ds_src(p, b, h, kh, s0 + ct, j0, cols, dimp, per, i);
+      if (i < nn) pf[u] = ds_src(p, b, h, kh, s0 + ct, j0, cols, dimp, per, per_magic, i);
     }
     for (int tt = 0; tt < nt; ++tt) {
       const float* row = stage + tt * per;
-      const float4* k4 = reinterpret_cast<const float4*>(row + i0);
-      const float4* q4 = reinterpret_cast<const float4*>(row + dimp + i0);
+      const float4* k4 = reinterpret_cast<const float4*>(row + r * DS_PITCH);
+      const float4* q4 = reinterpret_cast<const float4*>(row + dimp + r * DS_PITCH);
       const float v = row[2 * dimp + jl], g = row[2 * dimp + cols], beta = row[2 * dimp + cols + 1];
       float kv[DS_SLICE], qv[DS_SLICE], sk0 = 0.f, sk1 = 0.f;
 #pragma unroll
@@ -232,11 +239,12 @@ int hy_delta_scan(const DeltaScan& p, hipStream_t s) {
   if (p.H > 65535 || p.B > 65535) return -3;
   int R = 1;
   while (R * DS_SLICE < p.dim) R <<= 1;
-  const int per = (2 * R * DS_SLICE + 256 / R + 2 + 3) / 4 * 4;
+  const int per = (2 * R * DS_PITCH + 256 / R + 2 + 3) / 4 * 4;
   if (per > DS_STAGE) return -4;
   const int ct = DS_STAGE / per < 32 ? DS_STAGE / per : 32;
   const long long threads = (long long)p.vdim * R;
-  delta_scan_kernel<<<dim3((unsigned)((threads + 255) / 256), p.H, p.B), 256, 0, s>>>(p, R, ct, per);
+  const unsigned per_magic = (unsigned)((0x100000000ull + per - 1) / per);  // ceil(2^32 / per)
+  delta_scan_kernel<<<dim3((unsigned)((threads + 255) / 256), p.H, p.B), 256, 0, s>>>(p, R, ct, per, per_magic);
   JLA_CHECK_LAUNCH();
   return 0;
 }
