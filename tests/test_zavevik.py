@@ -399,3 +399,20 @@ def test_longer_prompts_at_the_mfma_head_sizes(dtype):
     assert max(e) < (2e-4 if dtype == F32 else 4e-2), (int(np.argmax(e)), max(e))
     whole = run_portions(model, t, [600])
     assert err(whole, got) < (2e-5 if dtype == F32 else 2e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_sampled_generation_through_the_engine(device):
+    """The framework's sampler (temperature, top-k, top-p, seeded Philox) on Zavevik logits: reproducible per seed,
+    different across seeds, tokens inside the vocabulary, and every token inside the top-k of the oracle's logits."""
+    model, sd = build(cfg_full(), device)
+    prompt = torch.tensor([toks(7, 61, seed=14)], dtype=torch.int32)
+    gc = dict(max_length=27, pad_token_id=0, do_sample=True, temperature=0.9, top_k=5, top_p=0.95)
+    a = model.generate(prompt, generation_config=GenerationConfig(seed=3, **gc)).sequences[0].cpu().tolist()
+    b = model.generate(prompt, generation_config=GenerationConfig(seed=3, **gc)).sequences[0].cpu().tolist()
+    c = model.generate(prompt, generation_config=GenerationConfig(seed=4, **gc)).sequences[0].cpu().tolist()
+    assert a == b and a != c and all(0 <= x < 61 for x in a + c)
+    ref, _ = oz.forward(cfg_full(), sd, a)
+    for i in range(7, 27):
+        row = ref[i - 1]
+        assert row[a[i]] >= np.sort(row)[-5] - 1e-4 * np.abs(row).max(), i
