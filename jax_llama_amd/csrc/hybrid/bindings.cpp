@@ -45,6 +45,17 @@ int wtype(const Tensor& t, const char* name) {
   return t.scalar_type() == torch::kBFloat16;
 }
 
+// a 2-d fp32 or bf16 view with unit inner stride (rows may be strided); *bf = 1 for bf16
+void* rows2d_any(const Tensor& t, const char* name, int64_t cols, int* ld, int* bf) {
+  TORCH_CHECK(t.is_cuda() && (t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kBFloat16) &&
+                  t.dim() == 2 && t.stride(1) == 1 && t.size(1) == cols && t.stride(0) >= cols,
+              "jax_llama_amd._C_hybrid: ", name, " must be a float32 / bfloat16 [rows, ", cols,
+              "] GPU view with unit inner stride");
+  *ld = (int)t.stride(0);
+  *bf = t.scalar_type() == torch::kBFloat16;
+  return t.data_ptr();
+}
+
 // a 2-d fp32 view with unit inner stride (rows may be strided)
 const float* rows2d(const Tensor& t, const char* name, int64_t cols, int* ld) {
   TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.dim() == 2 && t.stride(1) == 1 &&
@@ -75,8 +86,8 @@ void linear_rows(Tensor a, OptT a_idx, Tensor w, Tensor out, OptT dst_idx, OptT 
   p.N = swiglu ? Nw / 2 : Nw;
   p.w = w.data_ptr();
   p.w_stride = Nw * (int64_t)p.K;
-  p.a = rows2d(a, "a", p.K, &p.lda);
-  p.out = const_cast<float*>(rows2d(out, "out", p.N, &p.ldo));
+  p.a = rows2d_any(a, "a", p.K, &p.lda, &p.a_bf16);
+  p.out = rows2d_any(out, "out", p.N, &p.ldo, &p.out_bf16);
   p.R = R;
   p.swiglu = swiglu;
   check(R >= 0, "linear_rows: R");

@@ -16,14 +16,16 @@ int hy_embed_rows(const int32_t* ids, const void* table, int wbf16, int V, int l
                   hipStream_t s);
 
 struct RowLinear {
-  const float* a;        // [*, lda] fp32 activations
+  const void* a;         // [*, lda] activations: fp32, or (a_bf16, tile path with bf16 weights only) bf16
+  int a_bf16;
   int lda;
   const int32_t* a_idx;  // optional: activation row of linear row r (else r)
   const void* w;         // [E][Nw][K] row-major; Nw = N (store) or 2N (swiglu: gate rows [0, N), up rows [N, 2N))
   long long w_stride;    // elements between experts
   int wbf16;
   int N, K;
-  float* out;            // [*, ldo] fp32
+  void* out;             // [*, ldo] fp32, or (out_bf16, tile path with bf16 weights only) bf16
+  int out_bf16;
   int ldo;
   const int32_t* dst_idx;     // optional: output row of linear row r (else r)
   const int32_t* offs;        // optional [E + 1]: rows [offs[e], offs[e + 1]) use expert e (rows sorted by expert)

@@ -3,8 +3,10 @@
 // A is fp32 in memory. With bf16 weights the A tile is rounded to bf16 while it is staged (v_mfma_f32_32x32x16_bf16,
 // fp32 accumulation); with fp32 weights everything stays fp32 on the exact-f32 MFMA (v_mfma_f32_32x32x2_f32).
 //
-//  * tiles: 64 x 64 outputs per 256-thread workgroup, four waves of 32 x 32, K staged 32 deep through LDS (several
-//    workgroups per CU hide each other's staging; a 128 x 128 tile with register prefetch and a 64-deep K stage measured slower). With an
+//  * tiles: 64 x 64 or (with rows to fill them) 128 x 64 outputs per 256-thread workgroup, four waves of 32 x 32 /
+//    64 x 32, K staged 32 deep through LDS (several workgroups per CU hide each other's staging; a 128 x 128 tile with
+//    register prefetch and a 64-deep K stage measured slower). The activations may be a bf16 copy and the output bf16
+//    (the expert pair of a prompt: x -> bf16 once, hidden kept bf16), which halves the activation traffic. With an
 //    expert offset table the m-tiles of the launch are dealt to the experts in order (a workgroup finds its expert by
 //    walking the table; surplus workgroups exit), so one launch covers every expert of a token-sorted batch.
 //  * few rows (decode): a wave streams one or four weight rows once and dots them with up to 8 activation rows.
@@ -50,22 +52,58 @@ JLA_DEV void lr_mma(const float* a_row, const float* b_row, int hi, f32x16& acc)
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_row[2 * kk + hi], b_row[2 * kk + hi], acc, 0, 0, 0);
 }
 
-template <typename WT, int SWIGLU>
+// 8 consecutive k of a row into the LDS tile (zeros past `left`); a bf16 source going to a bf16 tile is copied as is
+JLA_DEV void lr_stage8(const float* src, int left, bf16_t* dst) {
+  float f[8];
+  hy_load8(src, left, f);
+  lr_store8(dst, f);
+}
+JLA_DEV void lr_stage8(const float* src, int left, float* dst) {
+  float f[8];
+  hy_load8(src, left, f);
+  lr_store8(dst, f);
+}
+JLA_DEV void lr_stage8(const bf16_t* src, int left, bf16_t* dst) {
+  if (left >= 8 && ((uintptr_t)src & 15) == 0) {
+    *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+  } else {
+    float f[8];
+    hy_load8(src, left, f);
+    lr_store8(dst, f);
+  }
+}
+JLA_DEV void lr_stage8(const bf16_t* src, int left, float* dst) {
+  float f[8];
+  hy_load8(src, left, f);
+  lr_store8(dst, f);
+}
+template <typename T>
+JLA_DEV void lr_zero8(T* dst) {
+  const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  lr_store8(dst, z);
+}
+JLA_DEV void lr_out(float* p, float v) { *p = v; }
+JLA_DEV void lr_out(bf16_t* p, float v) { *p = f2bf(v); }
+
+// WT: weight / tile type; AT: activation type in memory (fp32, or a bf16 copy); OT: output type; TMM: 32-row tiles per
+// wave along M (workgroup tile 64 TMM x 64: the 128-row form halves the weight traffic per output row).
+template <typename WT, int SWIGLU, typename AT, typename OT, int TMM>
 __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
   constexpr int LD = LrTile<WT>::LD;
-  __shared__ __attribute__((aligned(16))) WT As[LR_BM * LD];
+  constexpr int BM = LR_BM * TMM;
+  __shared__ __attribute__((aligned(16))) WT As[BM * LD];
   __shared__ __attribute__((aligned(16))) WT Bs[(SWIGLU ? 2 : 1) * LR_BN * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, hi = lane >> 5;
   // which expert and which rows
-  int e = 0, r0 = blockIdx.y * LR_BM, rend = p.R;
+  int e = 0, r0 = blockIdx.y * BM, rend = p.R;
   if (p.offs) {
     int tile = blockIdx.y;
     bool found = false;
     for (e = 0; e < p.E; ++e) {
-      const int b = p.offs[e], cnt = p.offs[e + 1] - b, nt = (cnt + LR_BM - 1) / LR_BM;
+      const int b = p.offs[e], cnt = p.offs[e + 1] - b, nt = (cnt + BM - 1) / BM;
       if (tile < nt) {
-        r0 = b + tile * LR_BM;
+        r0 = b + tile * BM;
         rend = b + cnt;
         found = true;
         break;
@@ -80,63 +118,61 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemm_kernel(RowLinear p) {
   const WT* W = reinterpret_cast<const WT*>(p.w) + (size_t)e * p.w_stride;
   const int K = p.K, N = p.N;
 
-  // staging role: 8 consecutive k of one row
+  // staging role: 8 consecutive k of row (tid >> 2) (+ 64 for the second half of a 128-row tile)
   const int srow = tid >> 2, skq = (tid & 3) * 8;
-  const int ar = r0 + srow;
-  const float* a_ptr = nullptr;
-  if (ar < rend) a_ptr = p.a + (size_t)(p.a_idx ? p.a_idx[ar] : ar) * p.lda;
+  const AT* a_ptr[TMM];
+#pragma unroll
+  for (int t = 0; t < TMM; ++t) {
+    const int ar = r0 + srow + 64 * t;
+    a_ptr[t] = ar < rend ? reinterpret_cast<const AT*>(p.a) + (size_t)(p.a_idx ? p.a_idx[ar] : ar) * p.lda : nullptr;
+  }
   const int wr = n0 + srow;
   const WT* w_ptr = wr < N ? W + (size_t)wr * K : nullptr;
   const WT* w2_ptr = (SWIGLU && wr < N) ? W + (size_t)(N + wr) * K : nullptr;
 
-  f32x16 acc, acc2;
+  f32x16 acc[TMM], acc2[TMM];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.f;
+  for (int t = 0; t < TMM; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = acc2[t][r] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += LR_BK) {
+    const int gk = k0 + skq, left = K - gk;
 #pragma unroll
-    for (int half = 0; half < LR_BK / 32; ++half) {  // a thread stages 8 k of its row per 32-wide half
-      const int kq = skq + 32 * half, gk = k0 + kq, left = K - gk;
-      float f[8];
-      if (a_ptr && left > 0) hy_load8(a_ptr + gk, left, f);
-      else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = 0.f;
-      }
-      lr_store8(&As[srow * LD + kq], f);
-      if (w_ptr && left > 0) hy_load8(w_ptr + gk, left, f);
-      else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = 0.f;
-      }
-      lr_store8(&Bs[srow * LD + kq], f);
-      if (SWIGLU) {
-        if (w2_ptr && left > 0) hy_load8(w2_ptr + gk, left, f);
-        else {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) f[i] = 0.f;
-        }
-        lr_store8(&Bs[(LR_BN + srow) * LD + kq], f);
-      }
+    for (int t = 0; t < TMM; ++t) {
+      if (a_ptr[t] && left > 0) lr_stage8(a_ptr[t] + gk, left, &As[(srow + 64 * t) * LD + skq]);
+      else lr_zero8(&As[(srow + 64 * t) * LD + skq]);
+    }
+    if (w_ptr && left > 0) lr_stage8(w_ptr + gk, left, &Bs[srow * LD + skq]);
+    else lr_zero8(&Bs[srow * LD + skq]);
+    if (SWIGLU) {
+      if (w2_ptr && left > 0) lr_stage8(w2_ptr + gk, left, &Bs[(LR_BN + srow) * LD + skq]);
+      else lr_zero8(&Bs[(LR_BN + srow) * LD + skq]);
     }
     __syncthreads();
-    const WT* a_row = &As[(wm * 32 + (lane & 31)) * LD];
     const WT* b_row = &Bs[(wn * 32 + (lane & 31)) * LD];
-    lr_mma(a_row, b_row, hi, acc);
-    if (SWIGLU) lr_mma(a_row, b_row + LR_BN * LD, hi, acc2);
+#pragma unroll
+    for (int t = 0; t < TMM; ++t) {
+      const WT* a_row = &As[(wm * 32 * TMM + 32 * t + (lane & 31)) * LD];
+      lr_mma(a_row, b_row, hi, acc[t]);
+      if (SWIGLU) lr_mma(a_row, b_row + LR_BN * LD, hi, acc2[t]);
+    }
     __syncthreads();
   }
   // C/D map of the 32 x 32 shapes: col = lane & 31, row = (r & 3) + 8 (r >> 2) + 4 (lane >> 5)
   const int col = n0 + wn * 32 + (lane & 31);
   if (col >= N) return;
+  OT* out = reinterpret_cast<OT*>(p.out);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = r0 + wm * 32 + (r & 3) + 8 * (r >> 2) + 4 * hi;
-    if (row < rend) {
-      const int drow = p.dst_idx ? p.dst_idx[row] : row;
-      p.out[(size_t)drow * p.ldo + col] = SWIGLU ? hy_silu(acc[r]) * acc2[r] : acc[r];
+  for (int t = 0; t < TMM; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = r0 + wm * 32 * TMM + 32 * t + (r & 3) + 8 * (r >> 2) + 4 * hi;
+      if (row < rend) {
+        const int drow = p.dst_idx ? p.dst_idx[row] : row;
+        lr_out(out + (size_t)drow * p.ldo + col, SWIGLU ? hy_silu(acc[t][r]) * acc2[t][r] : acc[t][r]);
+      }
     }
-  }
 }
 
 JLA_DEV float lr_round(float v, const bf16_t*) { return bf2f(f2bf(v)); }
@@ -173,7 +209,7 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
     const int rr = r0 + min(r, nr - 1);
-    a[r] = p.a + (size_t)(p.a_idx ? p.a_idx[rr] : rr) * p.lda;
+    a[r] = reinterpret_cast<const float*>(p.a) + (size_t)(p.a_idx ? p.a_idx[rr] : rr) * p.lda;
   }
   float acc[MAXR][LR_CPW], acc2[MAXR][LR_CPW];
 #pragma unroll
@@ -214,7 +250,8 @@ __global__ void __launch_bounds__(LR_THREADS) lr_gemv_kernel(RowLinear p, int ro
       for (int c = 0; c < LR_CPW; ++c) {
         const float g = wave_sum(acc[r][c]);
         const float u = SWIGLU ? wave_sum(acc2[r][c]) : 0.f;
-        if (lane == 0 && n0 + c < p.N) p.out[(size_t)drow * p.ldo + n0 + c] = SWIGLU ? hy_silu(g) * u : g;
+        if (lane == 0 && n0 + c < p.N)
+          reinterpret_cast<float*>(p.out)[(size_t)drow * p.ldo + n0 + c] = SWIGLU ? hy_silu(g) * u : g;
       }
     }
   }
@@ -231,6 +268,7 @@ int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   const bool grouped = p.offs && p.R <= HY_GROUPED_GEMV_MAX_R;
   const bool small = grouped || (p.R <= HY_GEMV_MAX_R && (!p.offs || p.row_expert));
   if (small) {
+    if (p.a_bf16 || p.out_bf16) return -7;  // (the GEMV reads and writes fp32)
     const int rpg = p.row_expert && !grouped ? 1 : HY_GEMV_MAX_R;
     const int cpw = p.N >= 8192 ? 4 : 1;
     dim3 grid((p.N + 4 * cpw - 1) / (4 * cpw), grouped ? p.E : (p.R + rpg - 1) / rpg);
@@ -253,18 +291,31 @@ int hy_linear_rows(const RowLinear& p, hipStream_t s) {
     return 0;
   }
   if (!p.offs && p.E != 1) return -3;
-  const long long mt = (p.R + LR_BM - 1) / LR_BM + (p.offs ? p.E : 0);
+  if ((p.a_bf16 || p.out_bf16) && !p.wbf16) return -5;
+  // 128-row tiles once every expert (or the whole batch) has rows to fill them
+  const int tmm = p.R >= (p.offs ? 128 * p.E : 256) ? 2 : 1;
+  const int bm = LR_BM * tmm;
+  const long long mt = (p.R + bm - 1) / bm + (p.offs ? p.E : 0);
   if (mt > 65535) return -4;
   dim3 grid((p.N + LR_BN - 1) / LR_BN, (unsigned)mt);
   RowLinear q = p;
   q.row_expert = nullptr;
+#define LR_GEMM(WT, SW, AT, OT)                                                           \
+  do {                                                                                    \
+    if (tmm == 2) lr_gemm_kernel<WT, SW, AT, OT, 2><<<grid, LR_THREADS, 0, s>>>(q);       \
+    else lr_gemm_kernel<WT, SW, AT, OT, 1><<<grid, LR_THREADS, 0, s>>>(q);                \
+  } while (0)
   if (p.wbf16) {
-    if (p.swiglu) lr_gemm_kernel<bf16_t, 1><<<grid, LR_THREADS, 0, s>>>(q);
-    else lr_gemm_kernel<bf16_t, 0><<<grid, LR_THREADS, 0, s>>>(q);
+    if (p.a_bf16 && p.out_bf16 && p.swiglu) LR_GEMM(bf16_t, 1, bf16_t, bf16_t);
+    else if (p.a_bf16 && !p.out_bf16 && !p.swiglu) LR_GEMM(bf16_t, 0, bf16_t, float);
+    else if (p.a_bf16 || p.out_bf16) return -6;  // (combinations nothing uses)
+    else if (p.swiglu) LR_GEMM(bf16_t, 1, float, float);
+    else LR_GEMM(bf16_t, 0, float, float);
   } else {
-    if (p.swiglu) lr_gemm_kernel<float, 1><<<grid, LR_THREADS, 0, s>>>(q);
-    else lr_gemm_kernel<float, 0><<<grid, LR_THREADS, 0, s>>>(q);
+    if (p.swiglu) LR_GEMM(float, 1, float, float);
+    else LR_GEMM(float, 0, float, float);
   }
+#undef LR_GEMM
   JLA_CHECK_LAUNCH();
   return 0;
 }

@@ -95,6 +95,7 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor, col0: int = 0, ncols: Opt
 # (N % 16 == 0, K % 32 == 0); the row-major kernel here serves every other case. JLA_HY_PACKED_GEMM=0: never.
 PACKED_GEMM = os.environ.get("JLA_HY_PACKED_GEMM", "1") != "0"
 PACKED_GEMM_MIN_M = 256
+GROUPED_GEMV_MAX_R = 64  # rows up to which an expert-sorted batch runs the expert-grouped GEMV (csrc: HY_GROUPED_GEMV_MAX_R)
 _PACKED = {}
 
 
@@ -159,11 +160,20 @@ def moe_table(x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, w_gu: tor
     idx = torch.empty(4 * r + e_n + 1, dtype=torch.int32, device=dev)
     row_expert, row_tok, sort_tok, sort_dst, offs = idx[:r], idx[r:2 * r], idx[2 * r:3 * r], idx[3 * r:4 * r], idx[4 * r:]
     e.route_table(ids.to(torch.int32).contiguous(), table, e_n, row_expert, row_tok, sort_tok, sort_dst, offs)
-    h = torch.empty(r, w_gu.shape[1] // 2, dtype=F32, device=dev)
     y = torch.empty(r, w_down.shape[1], dtype=F32, device=dev)
+    bf16_pair = w_gu.dtype == BF16 and r > GROUPED_GEMV_MAX_R and x.is_contiguous() and x.shape[1] % 8 == 0
+    h = None if bf16_pair else torch.empty(r, w_gu.shape[1] // 2, dtype=F32, device=dev)
     if r <= e.GEMV_MAX_R:  # decode: one GEMV per (token, choice) row, expert read on the device
         e.linear_rows(x, row_tok, w_gu, h, None, None, row_expert, r, True)
         e.linear_rows(h, None, w_down, y, None, None, row_expert, r, False)
+    elif bf16_pair:
+        # prompt-sized, bf16: the tiles read a bf16 copy of x and keep the hidden activation bf16 (the operands they
+        # would round to anyway), which halves the activation traffic of both products
+        xb = torch.empty(x.shape, dtype=BF16, device=dev)
+        e.cast_bf16(x, xb)
+        hb = torch.empty(r, w_gu.shape[1] // 2, dtype=BF16, device=dev)
+        e.linear_rows(xb, sort_tok, w_gu, hb, None, offs, None, r, True)
+        e.linear_rows(hb, None, w_down, y, sort_dst, offs, None, r, False)
     else:  # expert-grouped tiles over the sorted rows; the down projection scatters back to (token, choice) order
         e.linear_rows(x, sort_tok, w_gu, h, None, offs, None, r, True)
         e.linear_rows(h, None, w_down, y, sort_dst, offs, None, r, False)
