@@ -292,8 +292,10 @@ int hy_linear_rows(const RowLinear& p, hipStream_t s) {
   }
   if (!p.offs && p.E != 1) return -3;
   if ((p.a_bf16 || p.out_bf16) && !p.wbf16) return -5;
-  // 128-row tiles once every expert (or the whole batch) has rows to fill them
-  const int tmm = p.R >= (p.offs ? 128 * p.E : 256) ? 2 : 1;
+  // 128-row tiles once every expert (or the whole batch) has rows to fill them; the SwiGLU form (two accumulator sets)
+  // only with many such tiles per expert (measured: 512 rows per expert run faster on 64-row tiles, 4096 on 128-row)
+  const long long per_e = p.R / (p.offs ? p.E : 1);
+  const int tmm = per_e >= (p.swiglu ? 1024 : (p.offs ? 128 : 256)) ? 2 : 1;
   const int bm = LR_BM * tmm;
   const long long mt = (p.R + bm - 1) / bm + (p.offs ? p.E : 0);
   if (mt > 65535) return -4;
