@@ -1,16 +1,20 @@
 """jax_llama_amd — an MI355X-native (gfx950 / CDNA4) LLaMA-1/2/3 inference framework with the
-public API of LSaldyt/JAX_llama (reference ``jax_llama/__init__.py:4-10``).
+public API of LSaldyt/JAX_llama (reference ``jax_llama/__init__.py:4-10``), plus a model registry with a second
+family (Zavevik: gated delta rule + biased attention + table-routed experts).
 
 Framework layer: PyTorch-ROCm. Hot path: hand-written HIP kernels (``csrc/kernels``).
 Multi-GPU: one process per GPU, RCCL + a custom xGMI all-reduce. Decode: hipGraph replay.
 """
-from .config import LLaMAConfig, ModelArgs, config_from_params, get_preset, swiglu_hidden_size
+from .config import LLaMAConfig, ModelArgs, ZavevikConfig, config_from_params, get_preset, swiglu_hidden_size
 from .generation import LLaMA
 from .models import (CausalLMOutput, FlaxLLaMAForCausalLM, FlaxLLaMAModel, KVCache, LLaMAForCausalLM,
                      LLaMAModel)
 from .parallel.partition import (Mesh, P, PartitionSpec, get_llama_param_partition_spec,
                                  with_named_sharding_constraint, with_sharding_constraint)
+from .models.registry import load_model
+from .models.zavevik import ZavevikForCausalLM
 from .runtime.engine import GenerationConfig
+from .runtime.stepper import SequenceStepper
 from .tokenizer import ChatFormat, LLaMA2Tokenizer, LLaMA3Tokenizer
 from .utils.checkpoint import convert_llama_weights
 
@@ -22,4 +26,5 @@ __all__ = [
     "CausalLMOutput", "KVCache", "GenerationConfig",
     "Mesh", "P", "PartitionSpec", "get_llama_param_partition_spec", "with_named_sharding_constraint",
     "with_sharding_constraint", "LLaMA2Tokenizer", "LLaMA3Tokenizer", "ChatFormat", "convert_llama_weights",
+    "ZavevikConfig", "ZavevikForCausalLM", "SequenceStepper", "load_model",
 ]
