@@ -23,7 +23,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..config import LayerSpec, MixerSpec, MoESpec, ZavevikConfig
+from ..config import MixerSpec, ZavevikConfig
 from ..ops import hybrid as hy
 from ..parallel.comm import NO_COMM
 from .kv_cache import HybridCache

@@ -2,8 +2,6 @@
 (tests/oracle_zavevik.py), on the CPU op path and, marked gpu, on the HIP kernels. Small configurations built here:
 sizes that are not multiples of any tile, unequal key / value widths, one and several lanes per recurrent column,
 top-1 / top-3 routing, a layer without feed-forward, shared keys, and a model without any of the optional parts."""
-import copy
-
 import numpy as np
 import pytest
 import torch
